@@ -12,7 +12,10 @@ __device__ __forceinline__ float gelu_tanh(float x) {
 
 template <int ACT>
 __global__ __launch_bounds__(256) void act_and_mul_kernel(const bf16* __restrict__ x, bf16* __restrict__ out,
-                                                          int64_t rows, int I, bool il, float limit) {
+                                                          int64_t rows, int I, bool il, float limit,
+                                                          const float* __restrict__ rg = nullptr,
+                                                          int64_t rg_stride = 0) {
+  // rg (optional): one fp32 logit per row, the row's output is multiplied by its sigmoid
   // grid (column blocks, rows): no per-element 64-bit division, every lane one 16-B vector.
   // il: gate / up columns interleaved in 16-column blocks (the layout of a gate_up weight
   // interleaved for the fused SiLU*mul GEMM epilogue, ops.interleave_gate_up)
@@ -24,6 +27,7 @@ __global__ __launch_bounds__(256) void act_and_mul_kernel(const bf16* __restrict
   const int gcol = il ? ((c * 8) >> 4) * 32 + ((c * 8) & 15) : c * 8;
   const int ucol = il ? gcol + 16 : I + c * 8;
   bf16x8 g = ld8(xr + gcol), u = ld8(xr + ucol), o;
+  const float rs = rg != nullptr ? 1.f / (1.f + expf(-rg[r * rg_stride])) : 1.f;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const float gf = (float)g[j];
@@ -33,10 +37,10 @@ __global__ __launch_bounds__(256) void act_and_mul_kernel(const bf16* __restrict
       const float L = limit > 0.f ? limit : (ACT == 2 ? 7.f : 20.f);
       const float g2 = fminf(gf, L);
       const float u2 = fminf(fmaxf((float)u[j], -L), L);
-      o[j] = (bf16)((u2 + 1.f) * g2 / (1.f + __expf(-1.702f * g2)));
+      o[j] = (bf16)((u2 + 1.f) * g2 / (1.f + __expf(-1.702f * g2)) * rs);
     } else {
       const float a = ACT == 0 ? silu(gf) : gelu_tanh(gf);
-      o[j] = (bf16)(a * (float)u[j]);
+      o[j] = (bf16)(a * (float)u[j] * rs);
     }
   }
   st8(out + r * I + c * 8, o);
@@ -72,7 +76,9 @@ static inline int grid_for(int64_t work, int nt) {
 // multiple of 8.  x [rows, 2I] = [gate | up].
 template <typename T>
 __global__ __launch_bounds__(256) void act_and_mul_any_kernel(const T* __restrict__ x, T* __restrict__ out,
-                                                              int I, int act, float limit) {
+                                                              int I, int act, float limit,
+                                                              const float* __restrict__ rg = nullptr,
+                                                              int64_t rg_stride = 0) {
   const int64_t r = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= I) return;
@@ -85,13 +91,14 @@ __global__ __launch_bounds__(256) void act_and_mul_any_kernel(const T* __restric
   } else {
     o = (act == 0 ? silu(gf) : gelu_tanh(gf)) * uf;
   }
+  if (rg != nullptr) o *= 1.f / (1.f + expf(-rg[r * rg_stride]));
   out[r * I + c] = (T)o;
 }
 
 // act: 0 SiLU, 1 GELU-tanh, 2 clamped SwiGLU (GPT-OSS: limit 7), 3 Phi-3-small GeGELU (limit 20);
 // limit > 0 replaces the clamp of act 2 / 3; | 16: interleaved gate/up (16-col blocks)
-OME_API int ome_act_and_mul(const void* x, void* out, int64_t rows, int I, int act, float limit,
-                            hipStream_t stream) {
+static int act_and_mul_launch(const void* x, void* out, int64_t rows, int I, int act, float limit, const float* rg,
+                              int64_t rg_stride, hipStream_t stream) {
   if (rows <= 0) return 0;
   const bool il = (act & 16) != 0, f32 = (act & 32) != 0;   // | 32: fp32 elements
   act &= 15;
@@ -103,10 +110,12 @@ OME_API int ome_act_and_mul(const void* x, void* out, int64_t rows, int I, int a
       const dim3 g((I + 255) / 256, (unsigned)n);
       if (f32)
         act_and_mul_any_kernel<float><<<g, 256, 0, stream>>>((const float*)x + r0 * 2 * I, (float*)out + r0 * I, I,
-                                                             act, limit);
+                                                             act, limit, rg ? rg + r0 * rg_stride : nullptr,
+                                                             rg_stride);
       else
         act_and_mul_any_kernel<bf16><<<g, 256, 0, stream>>>((const bf16*)x + r0 * 2 * I, (bf16*)out + r0 * I, I,
-                                                            act, limit);
+                                                            act, limit, rg ? rg + r0 * rg_stride : nullptr,
+                                                            rg_stride);
     }
     OME_CHECK_LAUNCH();
     return 0;
@@ -116,15 +125,52 @@ OME_API int ome_act_and_mul(const void* x, void* out, int64_t rows, int I, int a
     const dim3 g((I / 8 + 255) / 256, (unsigned)n);
     const bf16* xp = (const bf16*)x + r0 * 2 * I;
     bf16* op = (bf16*)out + r0 * I;
+    const float* rgp = rg ? rg + r0 * rg_stride : nullptr;
     if (act == 0)
-      act_and_mul_kernel<0><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
+      act_and_mul_kernel<0><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit, rgp, rg_stride);
     else if (act == 1)
-      act_and_mul_kernel<1><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
+      act_and_mul_kernel<1><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit, rgp, rg_stride);
     else if (act == 2)
-      act_and_mul_kernel<2><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
+      act_and_mul_kernel<2><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit, rgp, rg_stride);
     else
-      act_and_mul_kernel<3><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit);
+      act_and_mul_kernel<3><<<g, 256, 0, stream>>>(xp, op, n, I, il, limit, rgp, rg_stride);
   }
+  OME_CHECK_LAUNCH();
+  return 0;
+}
+
+OME_API int ome_act_and_mul(const void* x, void* out, int64_t rows, int I, int act, float limit,
+                            hipStream_t stream) {
+  return act_and_mul_launch(x, out, rows, I, act, limit, nullptr, 0, stream);
+}
+
+// row_gate: fp32 logits, one per row (rows row_gate_stride apart): row r of the output is also
+// multiplied by sigmoid(row_gate[r]) (a per-token gate on an always-on expert, applied ahead of
+// its down projection, which is linear).
+OME_API int ome_act_and_mul_rowgate(const void* x, void* out, int64_t rows, int I, int act, float limit,
+                                    const float* row_gate, int64_t row_gate_stride, hipStream_t stream) {
+  return act_and_mul_launch(x, out, rows, I, act, limit, row_gate, row_gate_stride, stream);
+}
+
+// Non-gated activation, any length and fp32 elements too (scalar accesses).
+template <typename T>
+__global__ __launch_bounds__(256) void act_any_kernel(T* __restrict__ x, int64_t n, int act) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const float f = (float)x[i];
+    x[i] = (T)(act == 0   ? f / (1.f + expf(-f))
+               : act == 1 ? gelu_tanh(f)
+               : act == 4 ? fmaxf(f, 0.f) * fmaxf(f, 0.f)
+               : act == 5 ? fmaxf(f, 0.f)
+                          : 0.5f * f * (1.f + erff(f * 0.7071067811865476f)));
+  }
+}
+
+OME_API int ome_act_any(void* x, int64_t n, int act, int f32, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (act != 0 && act != 1 && act != 3 && act != 4 && act != 5) return -3;
+  const int g = grid_for(n, 256);
+  if (f32) act_any_kernel<float><<<g, 256, 0, stream>>>((float*)x, n, act);
+  else act_any_kernel<bf16><<<g, 256, 0, stream>>>((bf16*)x, n, act);
   OME_CHECK_LAUNCH();
   return 0;
 }

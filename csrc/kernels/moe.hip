@@ -26,6 +26,8 @@
 // 2 = DeepSeek-V3 "noaux_tc" (group score = sum of the group's top-2 biased scores).  Experts are
 // chosen on score + bias (``e_score_correction_bias``) restricted to the best ``topk_group``
 // groups (other experts score 0, as in the HF reference); weights are the unbiased scores.
+// 3 = group score = max like 1, but experts outside the chosen groups count as minus infinity (never
+// chosen while an allowed expert is left, however negative the biased scores are).
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ logits, int64_t stride, int n_tok,
                                                         int E, int k, int renorm, int scoring,
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
     const int e = lane + 64 * i;
-    key[i] = e < E ? v[i] + (bias ? bias[e] : 0.f) : -3.f;
+    key[i] = e < E ? v[i] + (bias ? bias[e] : 0.f) : OME_NEG_INF;
   }
   if (group_mode && n_group > 1) {
     const int gs = E / n_group;
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
           b2 = x;
         }
       }
-      gscore = group_mode == 1 ? b1 : b1 + (gs > 1 ? b2 : 0.f);
+      gscore = group_mode == 2 ? b1 + (gs > 1 ? b2 : 0.f) : b1;
     }
     int chosen = 0;  // bit set on the lanes whose group is selected
     for (int j = 0; j < topk_group; ++j) {
@@ -114,18 +116,20 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
 #pragma unroll
     for (int i = 0; i < MAXV; ++i) {
       const int e = lane + 64 * i;
-      if (e < E && !s_gsel[wave][e / gs]) key[i] = 0.f;
+      if (e < E && !s_gsel[wave][e / gs]) key[i] = group_mode == 3 ? OME_NEG_INF : 0.f;
     }
   }
   float picked_sum = 0.f;
+  unsigned taken = 0;   // bit i: this lane's expert lane + 64 i was chosen already
   for (int j = 0; j < k; ++j) {
-    // argmax over the wave on the selection key (ties -> lowest expert id)
-    float best = -4.f, bw = 0.f;
+    // argmax over the wave on the selection key (ties -> lowest expert id); keys may be any
+    // finite value or minus infinity (masked groups), NaN keys are never picked
+    float best = OME_NEG_INF, bw = 0.f;
     int bi = 1 << 30;
 #pragma unroll
     for (int i = 0; i < MAXV; ++i) {
       const int e = lane + 64 * i;
-      if (e < E && (key[i] > best || (key[i] == best && e < bi))) {
+      if (e < E && !((taken >> i) & 1u) && (key[i] > best || (key[i] == best && e < bi))) {
         best = key[i];
         bw = v[i];
         bi = e;
@@ -153,7 +157,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
     picked_sum += bw;
 #pragma unroll
     for (int i = 0; i < MAXV; ++i)  // remove the winner (static register indexing)
-      if (lane + 64 * i == bi) key[i] = -5.f;
+      if (lane + 64 * i == bi) taken |= 1u << i;
   }
   if (renorm && lane == 0) {
     const float inv = 1.f / (picked_sum + 1e-20f);

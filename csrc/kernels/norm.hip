@@ -665,3 +665,114 @@ OME_API int ome_row_norm(const void* x, int64_t x_stride, int x_f32, const void*
   OME_CHECK_LAUNCH();
   return 0;
 }
+
+// ------------------------------------------------------------------------------------------
+// Pre-norm step of an fp32 residual stream with a token shift.  For row t of sequence s:
+//   v[t]   = res_in[t] + s1 * x1[t] + s2 * x2[t]            (either addend may be absent)
+//   n[t]   = v[t] / sqrt(mean(v[t]^2) + eps) * (w_off + w)  (fp32; w_off = 1 for weights stored
+//                                                            as the offset from one)
+//   out[t] = n[t] + (n[t-1] - n[t]) * mu                     (rounded once, to T)
+// n[t-1] of a sequence's first row of this step is the row kept per request slot in `state`
+// [slots, H] fp32 (zeros when reset[s] is set); the step's last n of the sequence replaces it.
+// The updated stream goes to a second buffer (res_out), so the workgroup of row t can form n[t-1]
+// from the step's inputs without waiting for the workgroup of row t-1.  Only the workgroup of a
+// sequence's first row touches the state: it reads the old row, then (after forming the n of the
+// sequence's last row itself) writes the new one.  mu == nullptr: no shift (plain norm, no state).
+// ------------------------------------------------------------------------------------------
+namespace {
+template <typename T>
+__device__ __forceinline__ float shift_row_rs(const float* __restrict__ r, const T* __restrict__ a, float s1,
+                                              const T* __restrict__ b, float s2, int H, float eps, float* red) {
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float v = r[i];
+    if (a != nullptr) v += s1 * (float)a[i];
+    if (b != nullptr) v += s2 * (float)b[i];
+    ss += v * v;
+  }
+  return 1.f / sqrtf(block_sum<256>(ss, red) / (float)H + eps);
+}
+
+template <typename T>
+__device__ __forceinline__ float shift_val(const float* r, const T* a, float s1, const T* b, float s2, int i) {
+  float v = r[i];
+  if (a != nullptr) v += s1 * (float)a[i];
+  if (b != nullptr) v += s2 * (float)b[i];
+  return v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void shift_norm_kernel(
+    const float* __restrict__ res_in, float* __restrict__ res_out, int64_t res_stride, const T* __restrict__ x1,
+    int64_t x1_stride, float s1, const T* __restrict__ x2, int64_t x2_stride, float s2, const T* __restrict__ w,
+    float w_off, const T* __restrict__ mu, float* __restrict__ state, const int* __restrict__ cu,
+    const int* __restrict__ slot, const int* __restrict__ reset, int S, T* __restrict__ out, int64_t out_stride,
+    int H, float eps) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const float* r = res_in + row * res_stride;
+  const T* a = x1 != nullptr ? x1 + row * x1_stride : nullptr;
+  const T* b = x2 != nullptr ? x2 + row * x2_stride : nullptr;
+  const float rs = shift_row_rs(r, a, s1, b, s2, H, eps, red);
+  float* ro = res_out + row * res_stride;
+  T* o = out + row * out_stride;
+  if (mu == nullptr) {
+    for (int i = threadIdx.x; i < H; i += 256) {
+      const float v = shift_val(r, a, s1, b, s2, i);
+      ro[i] = v;
+      o[i] = (T)(v * rs * (w_off + (float)w[i]));
+    }
+    return;
+  }
+  int s = 0;
+  while (s + 1 < S && cu[s + 1] <= (int)row) ++s;   // the sequence with cu[s] <= row < cu[s + 1]
+  const int first = cu[s], last = cu[s + 1] - 1;
+  if ((int)row != first) {   // the row before belongs to this step
+    const float* rp = r - res_stride;
+    const T* ap = a != nullptr ? a - x1_stride : nullptr;
+    const T* bp = b != nullptr ? b - x2_stride : nullptr;
+    const float rsp = shift_row_rs(rp, ap, s1, bp, s2, H, eps, red);
+    for (int i = threadIdx.x; i < H; i += 256) {
+      const float v = shift_val(r, a, s1, b, s2, i), wi = w_off + (float)w[i];
+      const float n = v * rs * wi, np = shift_val(rp, ap, s1, bp, s2, i) * rsp * wi;
+      ro[i] = v;
+      o[i] = (T)(n + (np - n) * (float)mu[i]);
+    }
+    return;
+  }
+  float* st = state + (int64_t)slot[s] * H;
+  const bool fresh = reset[s] != 0;
+  const int64_t d = last - first;   // rows from this one to the sequence's last of the step
+  const float* rl = r + d * res_stride;
+  const T* al = a != nullptr ? a + d * x1_stride : nullptr;
+  const T* bl = b != nullptr ? b + d * x2_stride : nullptr;
+  const float rsl = d > 0 ? shift_row_rs(rl, al, s1, bl, s2, H, eps, red) : rs;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float v = shift_val(r, a, s1, b, s2, i), wi = w_off + (float)w[i];
+    const float n = v * rs * wi, np = fresh ? 0.f : st[i];
+    ro[i] = v;
+    o[i] = (T)(n + (np - n) * (float)mu[i]);
+    st[i] = d > 0 ? shift_val(rl, al, s1, bl, s2, i) * rsl * wi : n;
+  }
+}
+}  // namespace
+
+OME_API int ome_shift_norm(const float* res_in, float* res_out, int64_t res_stride, const void* x1, int64_t x1_stride,
+                           float s1, const void* x2, int64_t x2_stride, float s2, const void* w, float w_off,
+                           const void* mu, float* state, const int* cu, const int* slot, const int* reset, int S,
+                           void* out, int64_t out_stride, int rows, int H, float eps, int f32, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || (mu != nullptr && (S <= 0 || state == nullptr))) return -2;
+  if (f32)
+    shift_norm_kernel<float><<<rows, 256, 0, stream>>>(res_in, res_out, res_stride, (const float*)x1, x1_stride, s1,
+                                                       (const float*)x2, x2_stride, s2, (const float*)w, w_off,
+                                                       (const float*)mu, state, cu, slot, reset, S, (float*)out,
+                                                       out_stride, H, eps);
+  else
+    shift_norm_kernel<bf16><<<rows, 256, 0, stream>>>(res_in, res_out, res_stride, (const bf16*)x1, x1_stride, s1,
+                                                      (const bf16*)x2, x2_stride, s2, (const bf16*)w, w_off,
+                                                      (const bf16*)mu, state, cu, slot, reset, S, (bf16*)out,
+                                                      out_stride, H, eps);
+  OME_CHECK_LAUNCH();
+  return 0;
+}

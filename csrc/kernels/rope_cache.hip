@@ -439,3 +439,192 @@ OME_API int ome_wide_norm_rope_cache(const void* q, int64_t q_stride, const void
   OME_CHECK_LAUNCH();
   return 0;
 }
+
+// ------------------------------------------------------------------------------------------
+// Attention input with short causal convolutions: q, k, v (row-strided views of one projection)
+// each pass a depthwise convolution over time (K taps per channel, no bias, no activation), then
+// q and k get the rotary embedding on the first rot_dim dims of every head (interleaved pairs
+// 2i / 2i+1, or halves i / i + rot_dim/2; angles from the fp32 cos | sin table row of the token's
+// position) and, AFTER the rotation, each head is divided by its root mean square over `dim`
+// (unit_norm; no weight).  q goes to q_out [T, Hq, D], k / v into the paged cache (K [pages, Hkv,
+// P, D], V [pages, Hkv, D, P]); head tails beyond dim / vdim are written as zeros (q, k) or left
+// as the cache's zeros (v).  Convolution sum, angles, rotation and norm are fp32; one rounding at
+// the store.
+//
+// The last K-1 projected rows of every sequence live in `tail` [slots, K-1, C] (C = all q, k, v
+// channels; row j = input at time -(K-1) + j of the next step).  Time is tiled: one workgroup =
+// (head of q / k / v, sequence, tile of CR_TILE rows); a wave owns a row at a time, lanes own the
+// head's channels.  Only a sequence's first tile touches the tail: it reads the old rows into LDS
+// and then writes the new ones from the step's last rows (or the shifted old rows of a step
+// shorter than K-1), so tiles never race.  K == 0: no convolution (and no tail).
+// ------------------------------------------------------------------------------------------
+namespace {
+constexpr int CR_TILE = 32;
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_rope_cache_kernel(
+    const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride, const T* __restrict__ v,
+    int64_t v_stride, const T* __restrict__ wq, const T* __restrict__ wk, const T* __restrict__ wv, int K,
+    T* __restrict__ tail, const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ reset,
+    const int* __restrict__ positions, const float* __restrict__ cos_sin, int rot_dim, int interleaved,
+    int unit_norm, float eps, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P) {
+  extern __shared__ float sm[];   // [CR_TILE + K - 1][d] input rows, then [K][d] taps
+  const int hh = blockIdx.x, s = blockIdx.y;
+  const int r0 = cu[s], r1 = cu[s + 1];
+  const int a = r0 + blockIdx.z * CR_TILE;
+  if (a >= r1) return;
+  const int e = min(a + CR_TILE, r1);
+  const int kind = hh < Hq ? 0 : (hh < Hq + Hkv ? 1 : 2);
+  const int head = kind == 0 ? hh : (kind == 1 ? hh - Hq : hh - Hq - Hkv);
+  const int d = kind == 2 ? vdim : dim;
+  const T* src = kind == 0 ? q : (kind == 1 ? k : v);
+  const int64_t sstride = kind == 0 ? q_stride : (kind == 1 ? k_stride : v_stride);
+  const T* wt = kind == 0 ? wq : (kind == 1 ? wk : wv);
+  const int C = Hq * dim + Hkv * dim + Hkv * vdim;
+  const int c0 = kind == 0 ? head * dim : (kind == 1 ? Hq * dim + head * dim : (Hq + Hkv) * dim + head * vdim);
+  const int KT = K > 0 ? K - 1 : 0;
+  float* rows = sm;
+  float* taps = sm + (CR_TILE + KT) * d;
+  const int tid = threadIdx.x;
+  for (int i = tid; i < K * d; i += 256) taps[i] = (float)wt[(int64_t)(head * d + i % d) * K + i / d];   // [j][c]
+  T* tl = KT > 0 ? tail + (int64_t)slot[s] * KT * C + c0 : nullptr;
+  const bool fresh = reset[s] != 0;
+  // input rows a - KT .. e - 1 of the sequence (before r0: the old tail, or zeros)
+  for (int i = tid; i < (e - a + KT) * d; i += 256) {
+    const int rr = i / d, c = i - rr * d;
+    const int r = a - KT + rr;
+    float x;
+    if (r >= r0) x = (float)src[(int64_t)r * sstride + head * d + c];
+    else x = fresh ? 0.f : (float)tl[(int64_t)(KT + (r - r0)) * C + c];
+    rows[rr * d + c] = x;
+  }
+  __syncthreads();
+  if (blockIdx.z == 0 && KT > 0) {   // new tail: inputs L - KT .. L - 1 of the step; negative = old tail rows
+    const int L = r1 - r0;
+    for (int i = tid; i < KT * d; i += 256) {
+      const int j = i / d, c = i - j * d;
+      const int t = L - KT + j;
+      tl[(int64_t)j * C + c] = t >= 0 ? src[(int64_t)(r0 + t) * sstride + head * d + c] : (T)rows[(KT + t) * d + c];
+    }
+  }
+  const int wave = tid >> 6, lane = tid & 63;
+  const int half = rot_dim >> 1;
+  for (int r = a + wave; r < e; r += 4) {
+    const int rr = r - a;   // output row rr reads input rows rr .. rr + KT
+    float y[4];             // channels lane, lane + 64, lane + 128, lane + 192 (d <= 256)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = lane + 64 * u;
+      float acc = 0.f;
+      if (c < d) {
+        if (K > 0)
+          for (int j = 0; j < K; ++j) acc += taps[j * d + c] * rows[(rr + j) * d + c];
+        else
+          acc = rows[rr * d + c];
+      }
+      y[u] = acc;
+    }
+    const int slot_t = slots[r];
+    if (kind == 2) {
+      if (slot_t >= 0) {
+        T* vc = v_cache + (((int64_t)(slot_t / P) * Hkv + head) * D) * P + slot_t % P;
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (lane + 64 * u < d) vc[(int64_t)(lane + 64 * u) * P] = (T)y[u];
+      }
+      continue;
+    }
+    if (rot_dim > 0) {
+      const float* cs = cos_sin + (int64_t)positions[r] * rot_dim;
+      if (interleaved) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = lane + 64 * u;
+          const float other = __shfl_xor(y[u], 1);
+          if (c < rot_dim) {
+            const float co = cs[c >> 1], si = cs[half + (c >> 1)];
+            y[u] = (c & 1) ? y[u] * co + other * si : y[u] * co - other * si;
+          }
+        }
+      } else {   // channel i pairs with i + half: the partner sits in lane pc & 63, register pc >> 6
+        float other[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = lane + 64 * u;
+          const int pc = c < half ? c + half : c - half;
+          float o = 0.f;
+#pragma unroll
+          for (int u2 = 0; u2 < 4; ++u2) {
+            const float cand = __shfl(y[u2], pc & 63);
+            if ((pc >> 6) == u2) o = cand;
+          }
+          other[u] = o;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = lane + 64 * u;
+          if (c < rot_dim) {
+            const int i = c < half ? c : c - half;
+            const float co = cs[i], si = cs[half + i];
+            y[u] = c < half ? y[u] * co - other[u] * si : y[u] * co + other[u] * si;
+          }
+        }
+      }
+    }
+    if (unit_norm) {
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) ss += (lane + 64 * u < d) ? y[u] * y[u] : 0.f;
+      const float rs = 1.f / sqrtf(wave_sum(ss) / (float)d + eps);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) y[u] *= rs;
+    }
+    T* dst;
+    if (kind == 0) dst = q_out + ((int64_t)r * Hq + head) * D;
+    else dst = slot_t >= 0 ? k_cache + (((int64_t)(slot_t / P) * Hkv + head) * P + slot_t % P) * D : nullptr;
+    if (dst != nullptr) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = lane + 64 * u;
+        if (c < D) dst[c] = c < d ? (T)y[u] : (T)0.f;
+      }
+    }
+  }
+}
+}  // namespace
+
+OME_API int ome_conv_rope_cache(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                                int64_t v_stride, const void* wq, const void* wk, const void* wv, int K, void* tail,
+                                const int* cu, const int* slot, const int* reset, int S, const int* positions,
+                                const float* cos_sin, int rot_dim, int interleaved, int unit_norm, float eps,
+                                void* q_out, void* k_cache, void* v_cache, const int* slots, int T, int Hq, int Hkv,
+                                int dim, int vdim, int D, int P, int f32, hipStream_t stream) {
+  if (T <= 0 || S <= 0) return 0;
+  if (dim <= 0 || vdim <= 0 || dim > D || vdim > D || D > 256 || K < 0 || K > 33 || rot_dim > dim || (rot_dim & 1))
+    return -2;
+  if (K > 0 && (wq == nullptr || wk == nullptr || wv == nullptr || (K > 1 && tail == nullptr))) return -2;
+  const int tiles = (T + CR_TILE - 1) / CR_TILE;
+  if (tiles > 65535 || S > 65535) return -3;
+  const int dmax = dim > vdim ? dim : vdim;
+  const size_t lds = (size_t)((CR_TILE + (K > 0 ? K - 1 : 0)) * dmax + K * dmax) * sizeof(float);
+  if (lds > 160 * 1024) return -3;
+  dim3 grid(Hq + 2 * Hkv, S, tiles);
+#define CRC_LAUNCH(TT)                                                                                              \
+  do {                                                                                                              \
+    if (lds > 64 * 1024) {                                                                                          \
+      hipError_t e_ = hipFuncSetAttribute((const void*)conv_rope_cache_kernel<TT>,                                  \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                    \
+      if (e_ != hipSuccess) return (int)e_;                                                                         \
+    }                                                                                                               \
+    conv_rope_cache_kernel<TT><<<grid, 256, lds, stream>>>(                                                         \
+        (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, (const TT*)wq, (const TT*)wk,       \
+        (const TT*)wv, K, (TT*)tail, cu, slot, reset, positions, cos_sin, rot_dim, interleaved, unit_norm, eps,     \
+        (TT*)q_out, (TT*)k_cache, (TT*)v_cache, slots, Hq, Hkv, dim, vdim, D, P);                                   \
+  } while (0)
+  if (f32) CRC_LAUNCH(float);
+  else CRC_LAUNCH(bf16);
+#undef CRC_LAUNCH
+  OME_CHECK_LAUNCH();
+  return 0;
+}

@@ -152,17 +152,37 @@ def latent_row_width(kv_rank: int, rot_dim: int) -> int:
     return -(-d // 64) * 64
 
 
+def layer_runs(c: dict[str, Any]) -> list[tuple[int, int]]:
+    """Execution order of a layer-list config as (layer, pass) pairs.  ``loop`` = {start, stop,
+    times}: layers start .. stop-1 run ``times`` times in a row (pass 0, 1, ...), every other layer
+    once; no ``loop``: every layer once."""
+    n = len(c["layers"])
+    lp = c.get("loop") or {}
+    times = int(lp.get("times", 1))
+    a, b = int(lp.get("start", 0)), int(lp.get("stop", 0))
+    if not lp or b <= a:
+        return [(i, 0) for i in range(n)]
+    if not (0 <= a < b <= n) or times < 0:
+        raise ValueError(f"loop {lp}: start / stop must lie within the {n} layers")
+    return [(i, 0) for i in range(a)] + [(i, p) for p in range(times) for i in range(a, b)] + \
+        [(i, 0) for i in range(b, n)]
+
+
 def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
-    """Layer-list configs (``architecture: Zavilorn`` / ``Metitar``): ``layers`` is a list of blocks,
-    each with its mixer ``type``, the mixer's own sizes and its feed-forward.  The standard keys
-    describe the envelope the runtime sizes its workspaces by (widest attention layer, fewest kv
-    heads); the model reads the per-layer entries from ``extra``."""
+    """Layer-list configs (``architecture: Zavilorn`` / ``Metitar`` / ``Milenex``): ``layers`` is a
+    list of blocks, each with its mixer ``type``, the mixer's own sizes and its feed-forward.  The
+    standard keys describe the envelope the runtime sizes its workspaces by (widest attention layer,
+    fewest kv heads); the model reads the per-layer entries from ``extra``.  ``num_hidden_layers``
+    counts layer RUNS (a looped span counts once per pass: every pass owns cache pages)."""
     attn, dims = [], []
     for L in c["layers"]:
         m = L.get("mixer") or {}
         if L.get("type") == "parallel":
             attn.append(m["left"])
             dims.append(attn_tile_dim(max(m["left"]["dim"], m["left"]["vdim"])))
+        elif L.get("type") in ("attention", "attention_2"):
+            attn.append(m)
+            dims.append(attn_tile_dim(max(m["dim"], m["vdim"])))
         elif L.get("type") == "latent_attention":   # absorbed form: one shared head of latent + rotary width
             attn.append(m)
             dims.append(latent_row_width(m["kv_rank"], m["rot_dim"]))
@@ -170,12 +190,13 @@ def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
     D = max(dims or [64])
     out = dict(c)
     out.update(architectures=[c["architecture"]], model_type=c["architecture"].lower(),
-               hidden_size=c["width"], vocab_size=c["vocab"], num_hidden_layers=len(c["layers"]),
+               hidden_size=c["width"], vocab_size=c["vocab"], num_hidden_layers=len(layer_runs(c)),
                rms_norm_eps=(c.get("norm") or {}).get("eps", 1e-6), tie_word_embeddings=True,
                num_attention_heads=max([a["heads"] for a in attn] or [1]),
                num_key_value_heads=min([a.get("kv_heads", 1) for a in attn] or [1]), head_dim=D,
-               intermediate_size=max(ff or [c["width"]]), rope_theta=(attn[0]["rot"]["base"] if attn else 10000.0),
-               partial_rotary_factor=(attn[0]["rot"]["dims"] / D if attn else 1.0),
+               intermediate_size=max(ff or [c["width"]]),
+               rope_theta=next((a["rot"]["base"] for a in attn if a.get("rot")), 10000.0),
+               partial_rotary_factor=next((a["rot"]["dims"] / D for a in attn if a.get("rot")), 1.0),
                max_position_embeddings=int(c.get("max_positions", 131072)), torch_dtype="bfloat16")
     return out
 

@@ -522,3 +522,210 @@ class TokenSideInput(_Block):
 
     def forward(self, h: torch.Tensor, ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
         return linear(ops.gelu_gather_mul(linear(h, self.w_gate), ids, table, self.col0), self.w_proj)
+
+
+def attention_rows(meta: AttnMeta, T: int) -> list:
+    """The step's rows for kernels that take one (block-table row, position) per query row:
+    segments (first row, end row, block table, block-table row per token, position per token) --
+    one for the prompt chunks, one for the single decode rows of a mixed step."""
+    return [(s, e, bt, rows, lens - 1) for s, e, bt, rows, lens in latent_rows(meta, T)]
+
+
+class ConvRotaryAttention(_Block):
+    """Grouped-query attention whose q, k and v each pass a short causal depthwise convolution
+    (``conv`` taps, no bias, no activation; 0: none) right after the projection; q and k are then
+    rotated on the first ``rot_dims`` dims of every head (interleaved or half-split pairs) and,
+    after the rotation, divided by their root mean square per head (no weight); score = q.k *
+    ``scale``; query i sees keys j with 0 <= i - j < ``window``; softmax whose denominator also
+    holds exp(``sink``_h); W_o.  Checkpoint tensors ``q k v [q.conv k.conv v.conv] sink o``;
+    state: the last conv - 1 projected rows per request slot."""
+
+    def __init__(self, layer: int, width: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int,
+                 conv: int, rot_base: float, rot_dims: int, scale: float, eps: float, max_positions: int, device,
+                 dtype, interleaved: bool = True, unit_norm: bool = True):
+        super().__init__(device, dtype)
+        if heads % kv_heads or heads // kv_heads > 16:
+            raise ValueError(f"attention: {heads} query heads over {kv_heads} kv heads (groups of <= 16 supported)")
+        self.layer, self.width, self.Hq, self.Hkv, self.dim, self.vdim = layer, width, heads, kv_heads, dim, vdim
+        self.window, self.K = int(window) if window and window > 0 else -1, int(conv or 0)
+        self.rot_dims, self.scale, self.eps = int(rot_dims), float(scale), float(eps)
+        self.interleaved, self.unit_norm = interleaved, unit_norm
+        self.D = attn_tile_dim(max(dim, vdim))
+        self.cos_sin = plain_rope_table(rot_base, self.rot_dims, max_positions, self.device) if rot_dims else \
+            torch.zeros(max_positions, 0, device=self.device)
+        self.nq, self.nk, self.nv = heads * dim, kv_heads * dim, kv_heads * vdim
+        self.w_in = self.cq = self.ck = self.cv = self.sink = self.w_o = None
+        self.tail = None
+
+    def load(self, t: dict) -> None:
+        self.w_in = self._put(torch.cat([t["q"], t["k"], t["v"]], 0))
+        if self.K:
+            self.cq, self.ck, self.cv = self._put(t["q.conv"]), self._put(t["k.conv"]), self._put(t["v.conv"])
+            for n, c, w in (("q", self.nq, self.cq), ("k", self.nk, self.ck), ("v", self.nv, self.cv)):
+                if tuple(w.shape) != (c, self.K):
+                    raise ValueError(f"{n}.conv: shape {tuple(w.shape)} != [{c}, {self.K}]")
+        self.sink, self.w_o = self._put(t["sink"], torch.float32), self._put(t["o"])
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_in = self._rand(gen, self.nq + self.nk + self.nv, self.width, std=std)
+        if self.K:
+            self.cq, self.ck, self.cv = (self._rand(gen, c, self.K, std=0.5) for c in (self.nq, self.nk, self.nv))
+        self.sink = torch.zeros(self.Hq, dtype=torch.float32, device=self.device)
+        self.w_o = self._rand(gen, self.width, self.Hq * self.vdim, std=std)
+
+    def alloc_state(self, slots: int) -> None:
+        if self.K > 1:
+            self.tail = torch.zeros(slots, self.K - 1, self.nq + self.nk + self.nv, dtype=self.dtype, device=self.device)
+
+    def forward(self, h: torch.Tensor, ctx: MixerCtx) -> torch.Tensor:
+        T = h.shape[0]
+        nq, nk = self.nq, self.nk
+        p = linear(h, self.w_in)                                   # [T, q | k | v]
+        q = torch.empty(T, self.Hq, self.D, dtype=h.dtype, device=h.device)
+        k_cache, v_cache = ctx.kv.layer(self.layer)
+        ops.conv_rope_cache(p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:], self.cq, self.ck, self.cv, self.tail, ctx.seqs,
+                            ctx.meta.positions, self.cos_sin, self.rot_dims, self.interleaved, self.unit_norm, self.eps,
+                            q, k_cache, v_cache, ctx.meta.slots, self.Hq, self.Hkv, self.dim, self.vdim)
+        a = paged_attention(q, k_cache, v_cache, ctx.meta, self.scale, self.window, 0, self.sink)
+        if self.D != self.vdim:
+            a = a[:, :, :self.vdim].reshape(T, self.Hq * self.vdim)
+        return linear(a.view(T, self.Hq * self.vdim), self.w_o)
+
+
+class TalkingHeadsAttention(_Block):
+    """Grouped-query attention without rotation: score = q.k * ``scale`` - r1_h ln(1 + r2_h (i -
+    j)) (a per-head logarithmic distance bias); query i sees keys j with 0 <= i - j < ``window``;
+    softmax whose denominator also holds exp(``sink``_h); the normalised weights are mixed across
+    heads (w_h <- sum_g talk[h, g] w_g) before head h applies them to the values of its own kv
+    head; every head's output is multiplied by sigmoid(W_g x)_h; W_o.  Checkpoint tensors ``q k v
+    r1 r2 talk sink g o``."""
+
+    def __init__(self, layer: int, width: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int,
+                 scale: float, device, dtype):
+        super().__init__(device, dtype)
+        if heads % kv_heads or heads // kv_heads > 16:
+            raise ValueError(f"attention: {heads} query heads over {kv_heads} kv heads (groups of <= 16 supported)")
+        if heads * vdim > 8192:
+            raise ValueError(f"talking-heads attention: {heads} heads x {vdim} value dims exceed 8192 outputs per row")
+        self.layer, self.width, self.Hq, self.Hkv, self.dim, self.vdim = layer, width, heads, kv_heads, dim, vdim
+        self.window, self.scale = int(window) if window and window > 0 else -1, float(scale)
+        self.D = attn_tile_dim(max(dim, vdim))
+        self.nq, self.nk, self.nv = heads * dim, kv_heads * dim, kv_heads * vdim
+        self.w_in = self.r1 = self.r2 = self.talk = self.sink = self.w_o = None
+        self._none = torch.zeros(1, 0, device=self.device)
+
+    def load(self, t: dict) -> None:
+        f32 = torch.float32
+        self.w_in = self._put(torch.cat([t["q"], t["k"], t["v"], t["g"]], 0))
+        self.r1, self.r2, self.talk = self._put(t["r1"], f32), self._put(t["r2"], f32), self._put(t["talk"], f32)
+        self.sink, self.w_o = self._put(t["sink"], f32), self._put(t["o"])
+        if tuple(self.talk.shape) != (self.Hq, self.Hq):
+            raise ValueError(f"talk: shape {tuple(self.talk.shape)} != [{self.Hq}, {self.Hq}]")
+
+    def init_random(self, gen, std: float) -> None:
+        f32 = dict(dtype=torch.float32, device=self.device)
+        H = self.Hq
+        self.w_in = self._rand(gen, self.nq + self.nk + self.nv + H, self.width, std=std)
+        self.r1, self.r2 = torch.linspace(0.1, 1.0, H, **f32), torch.linspace(0.5, 2.0, H, **f32)
+        self.talk = torch.eye(H, **f32) + 0.1 * torch.randn(H, H, generator=gen, **f32)
+        self.sink = torch.zeros(H, **f32)
+        self.w_o = self._rand(gen, self.width, H * self.vdim, std=std)
+
+    def forward(self, h: torch.Tensor, ctx: MixerCtx) -> torch.Tensor:
+        T = h.shape[0]
+        nq, nk, nv = self.nq, self.nk, self.nv
+        p = linear(h, self.w_in)                                   # [T, q | k | v | gate]
+        q = torch.empty(T, self.Hq, self.D, dtype=h.dtype, device=h.device)
+        k_cache, v_cache = ctx.kv.layer(self.layer)
+        ops.wide_norm_rope_cache(p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:nq + nk + nv], ctx.meta.positions,
+                                 self._none, 0, True, None, None, 0.0, q, k_cache, v_cache, ctx.meta.slots, self.Hq,
+                                 self.Hkv, self.dim, self.vdim)
+        o = torch.empty(T, self.Hq * self.vdim, dtype=h.dtype, device=h.device)
+        gate = p[:, nq + nk + nv:]
+        for s, e, bt, rows, pos in attention_rows(ctx.meta, T):
+            ops.talking_attn(q[s:e], k_cache, v_cache, bt, rows, pos, self.scale, self.window, self.sink, self.r1,
+                             self.r2, self.talk, gate[s:e], self.vdim, out=o[s:e])
+        return linear(o, self.w_o)
+
+
+class GeluMLP(_Block):
+    """W_down gelu(W_up h) with the exact (erf) GELU.  Checkpoint tensors ``up down``."""
+
+    def __init__(self, width: int, ff: int, device, dtype):
+        super().__init__(device, dtype)
+        self.width, self.ff = width, ff
+        self.w_up = self.w_d = None
+
+    def load(self, t: dict) -> None:
+        self.w_up, self.w_d = self._put(t["up"]), self._put(t["down"])
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_up, self.w_d = self._rand(gen, self.ff, self.width, std=std), self._rand(gen, self.width, self.ff,
+                                                                                        std=std)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return linear(ops.act(linear(h, self.w_up).contiguous(), 3), self.w_d)
+
+
+class GroupRoutedMoE(_Block):
+    """Mixture of clamped-GLU experts (:class:`ClampedGLU`'s form, no biases).  Router scores s =
+    softmax(W_r h) over all experts from fp32 logits; the choice is made on s + ``correction``,
+    among the experts of the ``keep`` best of ``groups`` equal groups of neighbours (a group scores
+    by its best choice score; experts of the other groups are excluded outright); the ``top``
+    chosen experts' outputs are weighted by their plain scores s (not renormalised).  An optional
+    shared expert (own width and ``limit``) runs for every token, times sigmoid(w_sg . h).
+    Checkpoint tensors ``router correction e<j>.gate|up|down [shared.gate|up|down|sg]``.
+
+    The router and the shared gate are one fp32-result GEMM (``[W_r; w_sg]``).  Experts run on the
+    grouped MFMA GEMMs (bf16, widths in multiples of 32), otherwise densely: every expert over all
+    rows as batched library GEMMs, weighted by the scattered scores (0 for unchosen experts) -- any
+    shape, fp32 models; no host synchronisation either way."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, groups: int, keep: int,
+                 shared_ff: int, shared_limit: float, device, dtype):
+        super().__init__(device, dtype)
+        if groups < 1 or experts % groups or not 1 <= keep <= groups or top > keep * (experts // groups):
+            raise ValueError(f"moe: {experts} experts in {groups} groups, {keep} kept, top {top}")
+        self.width, self.E, self.k, self.ff, self.limit = width, experts, top, ff, float(limit)
+        self.groups, self.keep = groups, keep
+        self.sff, self.slimit = int(shared_ff or 0), float(shared_limit or 0.0)
+        self.w_router = self.correction = self.w13 = self.w2 = self.w_sgu = self.w_sd = None
+
+    def load(self, t: dict) -> None:
+        self.w_router = self._put(torch.cat([t["router"], t["shared.sg"].reshape(1, -1)], 0) if self.sff
+                                  else t["router"])
+        self.correction = self._put(t["correction"], torch.float32)
+        self.w13 = self._put(torch.stack([torch.cat([t[f"e{e}.gate"], t[f"e{e}.up"]], 0) for e in range(self.E)]))
+        self.w2 = self._put(torch.stack([t[f"e{e}.down"] for e in range(self.E)]))
+        if self.sff:
+            self.w_sgu, self.w_sd = self._put(torch.cat([t["shared.gate"], t["shared.up"]], 0)), self._put(t["shared.down"])
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_router = self._rand(gen, self.E + (1 if self.sff else 0), self.width, std=std)
+        self.correction = torch.zeros(self.E, dtype=torch.float32, device=self.device)
+        self.w13, self.w2 = self._rand(gen, self.E, 2 * self.ff, self.width, std=std), self._rand(
+            gen, self.E, self.width, self.ff, std=std)
+        if self.sff:
+            self.w_sgu, self.w_sd = self._rand(gen, 2 * self.sff, self.width, std=std), self._rand(
+                gen, self.width, self.sff, std=std)
+
+    def grouped_ok(self, h: torch.Tensor) -> bool:
+        return h.is_cuda and h.dtype == torch.bfloat16 and self.width % 32 == 0 and self.ff % 32 == 0
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        T, W = h.shape
+        logits = ops.lm_head_f32(h, self.w_router)                        # fp32 [T, E (+ shared gate)]
+        tw, tid = ops.moe_route(logits[:, :self.E], self.k, False, "softmax", bias=self.correction,
+                                n_group=self.groups, topk_group=self.keep, group_mode=3 if self.groups > 1 else 0)
+        sh = None
+        if self.sff:
+            a = ops.act_and_mul(linear(h, self.w_sgu).contiguous(), 2, limit=self.slimit, row_gate=logits[:, self.E])
+            sh = linear(a, self.w_sd)
+        if self.grouped_ok(h):
+            return ops.fused_moe(h, tw, tid, self.w13, self.w2, act=2, limit=self.limit,
+                                 add=sh.contiguous() if sh is not None else None)
+        wd = torch.zeros(T, self.E, dtype=torch.float32, device=h.device).scatter_(1, tid.long(), tw)
+        gu = torch.matmul(h, self.w13.transpose(1, 2))                    # [E, T, 2 ff]
+        hh = ops.act_and_mul(gu.view(self.E * T, 2 * self.ff), 2, limit=self.limit).view(self.E, T, self.ff)
+        y = (torch.bmm(hh, self.w2.transpose(1, 2)).float() * wd.t()[:, :, None]).sum(0)
+        return (y if sh is None else y + sh.float()).to(h.dtype)

@@ -116,7 +116,11 @@ def act(x: torch.Tensor, kind: int) -> torch.Tensor:
     """In place non-gated activation: 0 SiLU, 1 GELU-tanh, 3 GELU (erf), 4 ReLU^2."""
     if not _gpu(x):
         return ref.act(x, kind)
-    assert x.is_contiguous() and x.dtype == torch.bfloat16
+    assert x.is_contiguous()
+    if x.dtype == torch.float32 or x.numel() % 8:   # fp32 models / odd lengths: the scalar kernel
+        call("ome_act_any", x.data_ptr(), x.numel(), int(kind), _f32(x), stream_ptr())
+        return x
+    assert x.dtype == torch.bfloat16
     call("ome_act", x.data_ptr(), x.numel(), int(kind), stream_ptr())
     return x
 
@@ -249,22 +253,29 @@ def kv_cache_write(k, v, k_cache, v_cache, slots, k_scale: float = 1.0, v_scale:
 
 
 def act_and_mul(x: torch.Tensor, act: int = 0, out: torch.Tensor | None = None,
-                interleaved: bool = False, limit: float = 0.0) -> torch.Tensor:
+                interleaved: bool = False, limit: float = 0.0, row_gate: torch.Tensor | None = None) -> torch.Tensor:
     """act 0 = SiLU (SwiGLU), 1 = GELU-tanh (GeGLU), 2 = GPT-OSS clamped SwiGLU, 3 = Phi-3-small
     GeGELU (quick-GELU gate, limit 20, ``up + 1``).  x [.., 2I] -> [.., I].  ``interleaved``:
     gate / up columns alternate in 16-column blocks (:func:`interleave_gate_up` weights).
-    ``limit`` > 0 replaces the clamp of act 2 / 3 (0: the family's constant)."""
+    ``limit`` > 0 replaces the clamp of act 2 / 3 (0: the family's constant).  ``row_gate``: fp32
+    logits, one per row (a strided [rows] view): row r of the output is also multiplied by
+    sigmoid(row_gate[r]) (a per-token gate on an always-on expert, ahead of its down projection)."""
     if not _gpu(x):
         if interleaved:
             g, u = deinterleave_gate_up(x.reshape(-1, x.shape[-1]))
             x = torch.cat([g, u], -1).view(*x.shape)
-        return ref.act_and_mul(x, act, limit)
+        return ref.act_and_mul(x, act, limit, row_gate)
     I = x.shape[-1] // 2
     rows = x.numel() // x.shape[-1]
     assert x.is_contiguous()
     out = torch.empty(*x.shape[:-1], I, dtype=x.dtype, device=x.device) if out is None else out
-    call("ome_act_and_mul", x.data_ptr(), out.data_ptr(), rows, I,
-         act | (16 if interleaved else 0) | (32 if _f32(x, out) else 0), float(limit), stream_ptr())
+    code = act | (16 if interleaved else 0) | (32 if _f32(x, out) else 0)
+    if row_gate is not None:
+        assert row_gate.dtype == torch.float32 and row_gate.dim() == 1 and row_gate.shape[0] == rows
+        call("ome_act_and_mul_rowgate", x.data_ptr(), out.data_ptr(), rows, I, code, float(limit),
+             row_gate.data_ptr(), row_gate.stride(0), stream_ptr())
+        return out
+    call("ome_act_and_mul", x.data_ptr(), out.data_ptr(), rows, I, code, float(limit), stream_ptr())
     return out
 
 
@@ -583,7 +594,9 @@ def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, scoring: str = 
               out_w: torch.Tensor | None = None, out_ids: torch.Tensor | None = None, bias: torch.Tensor | None = None,
               n_group: int = 1, topk_group: int = 1, group_mode: int = 0):
     """Router: logits [T, E] -> (weights f32 [T, k], expert ids int32 [T, k]).  ``group_mode`` 1/2 =
-    DeepSeek-V2 group_limited_greedy / DeepSeek-V3 noaux_tc (with ``bias``)."""
+    DeepSeek-V2 group_limited_greedy / DeepSeek-V3 noaux_tc (with ``bias``); 3 = a group scores by
+    its best biased expert and the experts of unchosen groups are excluded outright (minus
+    infinity where modes 1 / 2 set them to 0, which a negative biased score would lose against)."""
     if not _gpu(logits):
         w, ids = ref.moe_route(logits, k, renorm, scoring, bias, n_group, topk_group, group_mode)
         if out_w is not None:
@@ -630,17 +643,19 @@ def moe_fp8_tile_m(rows: int, E: int) -> int:
 
 def fused_moe(x: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor,
               act: int = 0, scale: float = 1.0, b13: torch.Tensor | None = None,
-              b2: torch.Tensor | None = None, gated: bool = True, add: torch.Tensor | None = None) -> torch.Tensor:
+              b2: torch.Tensor | None = None, gated: bool = True, add: torch.Tensor | None = None,
+              limit: float = 0.0) -> torch.Tensor:
     """Sparse MoE MLP on MFMA: align (counting sort by expert, on device) -> grouped GEMM gate_up
     with gathered A rows -> SiLU*mul -> grouped GEMM down -> weighted combine.  Shapes are
     static given T (graph-capturable); per-expert counts never leave the GPU.  ``gated=False``:
     w13 holds only up rows [E, I, H] and the activation is applied in place (NemotronH ReLU^2).
     ``add`` [T, H] (an always-on shared expert's output): returned as add + MoE, summed inside
-    the combine kernel (written into ``add`` itself)."""
+    the combine kernel (written into ``add`` itself).  ``limit`` > 0: the clamp of the clamped
+    activations (act 2 / 3) instead of the family's constant."""
     if hasattr(w13, "scale") and hasattr(w13, "q"):   # Fp8Experts (models/quant.py)
         return fused_moe_fp8(x, topk_w, topk_ids, w13, w2, act, scale, add=add)
     if not _gpu(x):
-        y = ref.fused_moe(x, topk_w, topk_ids, w13, w2, act, scale, b13, b2, gated)
+        y = ref.fused_moe(x, topk_w, topk_ids, w13, w2, act, scale, b13, b2, gated, limit)
         return y if add is None else add.copy_((add.float() + y.float()).to(add.dtype))
     T, H = x.shape
     E, I2, _ = w13.shape
@@ -657,7 +672,7 @@ def fused_moe(x: torch.Tensor, topk_w: torch.Tensor, topk_ids: torch.Tensor, w13
     gu = torch.empty(n, I2, dtype=x.dtype, device=dev)
     call("ome_moe_gemm", x.data_ptr(), x.stride(0), sorted_ids.data_ptr(), k, w13.data_ptr(), offsets.data_ptr(),
          E, I2, H, -(-n // tm) + E, gu.data_ptr(), gu.stride(0), ptr(b13), tm, stream_ptr())
-    h = act_and_mul(gu, act) if gated else _act_inplace(gu, act)
+    h = act_and_mul(gu, act, limit=limit) if gated else _act_inplace(gu, act)
     y = torch.empty(n, H, dtype=x.dtype, device=dev)
     tm = moe_tile_m(n, E, H)
     call("ome_moe_gemm", h.data_ptr(), h.stride(0), None, 0, w2.data_ptr(), offsets.data_ptr(), E, H, I,
@@ -1889,4 +1904,111 @@ def row_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, eps: floa
     out = torch.empty(x.shape, dtype=w.dtype, device=x.device)
     call("ome_row_norm", x.data_ptr(), x.stride(0), int(x.dtype == torch.float32), w.data_ptr(), ptr(b),
          out.data_ptr(), out.stride(0), x.shape[0], x.shape[1], float(eps), int(kind), f32, stream_ptr())
+    return out
+
+
+def shift_norm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor | None = None, s1: float = 1.0,
+               x2: torch.Tensor | None = None, s2: float = 1.0, w_offset: float = 0.0,
+               shift: torch.Tensor | None = None, state: torch.Tensor | None = None, seqs: tuple | None = None,
+               out_dtype=None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Pre-norm step of an fp32 residual stream, optionally with a token shift.  ``v = res + s1 x1 +
+    s2 x2`` (either addend may be None), ``n = v / sqrt(mean(v^2) + eps) * (w_offset + w)`` (``w_offset``
+    = 1 for weights stored as the offset from one), and with ``shift`` [H]: ``out[t] = n[t] +
+    (n[t-1] - n[t]) * shift`` where the row before a sequence's first row of the step is ``state[slot]``
+    ([slots, H] fp32; zeros when the sequence starts) and the sequence's last n replaces it
+    (``seqs`` = (cu, slot, reset)).  Sum, mean square, scaling and shift are fp32 with one rounding
+    at the end.  Returns (v, out): with a shift v is a NEW tensor (a row's workgroup also reads the
+    inputs of the row before it), without one ``res`` is updated in place and returned."""
+    if not _gpu(res):
+        v, out = ref.shift_norm(res, w, eps, x1, s1, x2, s2, w_offset, shift, state, seqs, out_dtype)
+        if shift is None:
+            res.copy_(v)
+            return res, out
+        return v, out
+    T, H = res.shape
+    assert res.dtype == torch.float32 and res.stride(1) == 1
+    if x2 is not None and x1 is None:
+        x1, s1, x2, s2 = x2, s2, None, 1.0
+    for a in (x1, x2):
+        assert a is None or (a.shape == res.shape and a.stride(1) == 1)
+    f32 = _f32(w, x1, x2, shift)
+    out = torch.empty(T, H, dtype=w.dtype, device=res.device)
+    if shift is not None:
+        cu, slot, reset = seqs
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1] == H and shift.shape[0] == H
+        new = torch.empty_like(res)
+        assert new.stride(0) == res.stride(0)
+        sargs = (shift.data_ptr(), state.data_ptr(), _i32(cu).data_ptr(), _i32(slot).data_ptr(),
+                 _i32(reset).data_ptr(), slot.shape[0])
+    else:
+        new, sargs = res, (None, None, None, None, None, 0)
+    call("ome_shift_norm", res.data_ptr(), new.data_ptr(), res.stride(0), ptr(x1),
+         x1.stride(0) if x1 is not None else 0, float(s1), ptr(x2), x2.stride(0) if x2 is not None else 0, float(s2),
+         w.data_ptr(), float(w_offset), *sargs, out.data_ptr(), out.stride(0), T, H, float(eps), f32, stream_ptr())
+    return new, out
+
+
+def conv_rope_cache(q, k, v, wq, wk, wv, tail, seqs, positions, cos_sin, rot_dim: int, interleaved: bool,
+                    unit_norm: bool, eps: float, q_out, k_cache, v_cache, slots, Hq: int, Hkv: int, dim: int,
+                    vdim: int) -> None:
+    """Attention input with short causal convolutions.  q [T, Hq*dim], k [T, Hkv*dim], v [T,
+    Hkv*vdim] (row-strided views of one projection) each pass a depthwise convolution over time
+    (taps ``wq`` / ``wk`` / ``wv`` [channels, K], no bias, no activation; all None: no
+    convolution); q and k are then rotated on the first ``rot_dim`` dims of every head
+    (``interleaved``: dim 2i pairs with 2i+1, else i with i + rot_dim/2; angles from the
+    ``cos_sin`` table row of the token's position) and -- ``unit_norm`` -- each head is divided by
+    its root mean square over ``dim`` AFTER the rotation (no weight).  q goes to ``q_out`` [T, Hq,
+    D], k / v into the paged cache at ``slots`` (head tails beyond dim / vdim are zero).  ``tail``
+    [slots, K-1, C] (C = all q, k, v channels, model dtype) keeps every sequence's last K-1
+    projected rows; ``seqs`` = (cu, slot, reset).  Convolution, rotation and norm are fp32."""
+    P, D = k_cache.shape[2], k_cache.shape[3]
+    assert dim <= D and vdim <= D and rot_dim <= dim and rot_dim % 2 == 0
+    if not _gpu(q):
+        return ref.conv_rope_cache(q, k, v, wq, wk, wv, tail, seqs, positions, cos_sin, rot_dim, interleaved, unit_norm,
+                                   eps, q_out, k_cache, v_cache, slots, Hq, Hkv, dim, vdim, P)
+    f32 = _f32(q, k, v, wq, wk, wv, tail, q_out, k_cache, v_cache)
+    cu, slot, reset = seqs
+    K = 0 if wq is None else wq.shape[1]
+    assert q_out.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert q.stride(1) == k.stride(1) == v.stride(1) == 1 and cos_sin.dtype == torch.float32
+    assert cos_sin.shape[1] == rot_dim or rot_dim == 0
+    if K:
+        assert tuple(wq.shape) == (Hq * dim, K) and tuple(wk.shape) == (Hkv * dim, K) and \
+            tuple(wv.shape) == (Hkv * vdim, K) and wq.is_contiguous() and wk.is_contiguous() and wv.is_contiguous()
+        assert K == 1 or (tail.is_contiguous() and tuple(tail.shape[1:]) == (K - 1, (Hq + Hkv) * dim + Hkv * vdim))
+    call("ome_conv_rope_cache", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+         ptr(wq), ptr(wk), ptr(wv), K, ptr(tail) if K > 1 else None, _i32(cu).data_ptr(), _i32(slot).data_ptr(),
+         _i32(reset).data_ptr(), slot.shape[0], _i32(positions).data_ptr(), cos_sin.data_ptr(), int(rot_dim),
+         int(bool(interleaved)), int(bool(unit_norm)), float(eps), q_out.data_ptr(), k_cache.data_ptr(),
+         v_cache.data_ptr(), _i32(slots).data_ptr(), q.shape[0], Hq, Hkv, dim, vdim, D, P, f32, stream_ptr())
+
+
+def talking_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                 row_seq: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int, sinks: torch.Tensor | None,
+                 r1: torch.Tensor, r2: torch.Tensor, talk: torch.Tensor, gate: torch.Tensor | None, vdim: int,
+                 out: torch.Tensor | None = None) -> torch.Tensor:
+    """Paged attention whose softmax weights are mixed across heads.  q [T, H, D] (D = the cache's
+    head width, zero beyond the key width); row t belongs to block-table row ``row_seq[t]`` at
+    position ``row_pos[t]`` (< 0: padding) and sees keys j with 0 <= pos - j < ``window`` (<= 0:
+    all).  score_g = q_g . k * scale - r1_g ln(1 + r2_g (pos - j)); w_g = softmax over the visible
+    keys with exp(``sinks``_g) added to the denominator; head h applies sum_g ``talk``[h, g] w_g to
+    the values of its own kv head; the result is multiplied by sigmoid(``gate``[t, h]) (a
+    row-strided [T, H] view, None: no gate).  Returns [T, H * vdim].  Prompt chunks and decode rows
+    are one launch; scores, weights and sums are fp32 for bf16 and fp32 models alike."""
+    T, H, D = q.shape
+    Hkv, P = k_cache.shape[1], k_cache.shape[2]
+    out = torch.empty(T, H * vdim, dtype=q.dtype, device=q.device) if out is None else out
+    if not _gpu(q):
+        return ref.talking_attn(q, k_cache, v_cache, block_tables, row_seq, row_pos, scale, window, sinks, r1, r2,
+                                talk, gate, vdim, out)
+    f32 = _f32(q, k_cache, v_cache, gate, out)
+    assert q.stride(2) == 1 and q.stride(1) == D and k_cache.shape[3] == D and out.stride(1) == 1
+    assert gate is None or gate.stride(1) == 1
+    for t in (r1, r2, talk):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    call("ome_talking_attn", q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+         _i32(block_tables).data_ptr(), block_tables.stride(0), _i32(row_seq.contiguous()).data_ptr(),
+         _i32(row_pos.contiguous()).data_ptr(), ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(),
+         out.stride(0), T, H, Hkv, D, vdim, P, float(scale), int(window), _sinks(sinks), r1.data_ptr(), r2.data_ptr(),
+         talk.data_ptr(), f32, stream_ptr())
     return out

@@ -56,6 +56,14 @@ _SIGNATURES = {
         "ome_latent_attn": [vp, i64, vp, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32, vp, i64, vp, vp, vp, vp],
         "ome_hgrn2_scan": [vp, vp, vp, i64, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp],
         "ome_act": [vp, i64, i32, vp],
+        "ome_act_any": [vp, i64, i32, i32, vp],
+        "ome_act_and_mul_rowgate": [vp, vp, i64, i32, i32, f32, vp, i64, vp],
+        "ome_shift_norm": [vp, vp, i64, vp, i64, f32, vp, i64, f32, vp, f32, vp, vp, vp, vp, vp, i32, vp, i64, i32,
+                           i32, f32, i32, vp],
+        "ome_conv_rope_cache": [vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32,
+                                f32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "ome_talking_attn": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i64, vp, i64, i32, i32, i32, i32, i32, i32, f32,
+                             i32, vp, vp, vp, vp, i32, vp],
         "ome_ssm_conv1d": [vp, i64, vp, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, vp],
         "ome_dyn_conv1d": [vp, i64, vp, i64, i32, vp, i64, vp, vp, vp, vp, i32, i32, i32, vp],
         "ome_qk_norm_rope": [vp, i64, vp, vp, i32, i32, i32, f32, vp, i64, vp, vp],

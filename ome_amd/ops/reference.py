@@ -229,16 +229,18 @@ def kv_cache_write(k, v, k_cache, v_cache, slots, P, k_scale=1.0, v_scale=1.0) -
     v_cache[page, :, :, off] = to_cache(v, v_cache.dtype, v_scale)
 
 
-def act_and_mul(x: torch.Tensor, act: int = 0, limit: float = 0.0) -> torch.Tensor:
+def act_and_mul(x: torch.Tensor, act: int = 0, limit: float = 0.0, row_gate=None) -> torch.Tensor:
+    """``row_gate`` (fp32 logits, one per row): the row's output is also multiplied by its sigmoid."""
     I = x.shape[-1] // 2
     g, u = x[..., :I].float(), x[..., I:].float()
+    rs = 1.0 if row_gate is None else torch.sigmoid(row_gate.float()).reshape(*x.shape[:-1], 1)
     if act in (2, 3):  # clamped SwiGLU / GeGELU: GPT-OSS (limit 7), Phi-3-small (limit 20)
         lim = float(limit) if limit and limit > 0 else (7.0 if act == 2 else 20.0)
         g = g.clamp(max=lim)
         u = u.clamp(-lim, lim)
-        return ((u + 1) * g * torch.sigmoid(1.702 * g)).to(x.dtype)
+        return ((u + 1) * g * torch.sigmoid(1.702 * g) * rs).to(x.dtype)
     a = torch.nn.functional.silu(g) if act == 0 else torch.nn.functional.gelu(g, approximate="tanh")
-    return (a * u).to(x.dtype)
+    return (a * u * rs).to(x.dtype)
 
 
 def embedding(ids: torch.Tensor, table: torch.Tensor, vocab_start: int = 0, vocab_end: int | None = None):
@@ -519,17 +521,18 @@ def pool(hidden, cu_lens, mode: int = 0, normalize: bool = True) -> torch.Tensor
 def moe_route(logits, k: int, renorm: bool, scoring: str = "softmax", bias=None, n_group: int = 1,
               topk_group: int = 1, group_mode: int = 0):
     """HF semantics (Mixtral/Qwen softmax top-k; DeepSeek-V2 group_limited_greedy = mode 1,
-    DeepSeek-V3 noaux_tc = mode 2 with e_score_correction_bias)."""
+    DeepSeek-V3 noaux_tc = mode 2 with e_score_correction_bias; mode 3 = the group's best
+    biased score, experts of the other groups excluded outright: minus infinity instead of 0)."""
     lf = logits.float()
     p = torch.softmax(lf, -1) if scoring == "softmax" else torch.sigmoid(lf)
     key = p + bias.float() if bias is not None else p.clone()
     if group_mode and n_group > 1:
         T, E = key.shape
         grp = key.view(T, n_group, E // n_group)
-        gs = grp.max(-1).values if group_mode == 1 else grp.topk(min(2, E // n_group), -1).values.sum(-1)
+        gs = grp.topk(min(2, E // n_group), -1).values.sum(-1) if group_mode == 2 else grp.max(-1).values
         gidx = gs.topk(topk_group, -1).indices
         gmask = torch.zeros_like(gs, dtype=torch.bool).scatter_(1, gidx, True)
-        key = key.masked_fill(~gmask.repeat_interleave(E // n_group, 1), 0.0)
+        key = key.masked_fill(~gmask.repeat_interleave(E // n_group, 1), float("-inf") if group_mode == 3 else 0.0)
     _, ids = torch.topk(key, k, dim=-1)  # ties: torch.topk order is implementation-defined
     w = p.gather(1, ids)
     if renorm:
@@ -537,7 +540,8 @@ def moe_route(logits, k: int, renorm: bool, scoring: str = "softmax", bias=None,
     return w.float(), ids.to(torch.int32)
 
 
-def fused_moe(x, topk_w, topk_ids, w13, w2, act: int = 0, scale: float = 1.0, b13=None, b2=None, gated=True):
+def fused_moe(x, topk_w, topk_ids, w13, w2, act: int = 0, scale: float = 1.0, b13=None, b2=None, gated=True,
+              limit: float = 0.0):
     """x [T, H]; w13 [E, 2I, H] (gate rows then up rows); w2 [E, H, I]; optional per-expert
     biases b13 [E, 2I], b2 [E, H] (GPT-OSS)."""
     T, H = x.shape
@@ -548,7 +552,7 @@ def fused_moe(x, topk_w, topk_ids, w13, w2, act: int = 0, scale: float = 1.0, b1
         gu = xf[tok] @ w13[e].float().t()
         if b13 is not None:
             gu = gu + b13[e].float()
-        h = (act_and_mul(gu.to(x.dtype), act) if gated else _act_inplace(gu.to(x.dtype), act)).float()
+        h = (act_and_mul(gu.to(x.dtype), act, limit) if gated else _act_inplace(gu.to(x.dtype), act)).float()
         y = h.to(x.dtype).float() @ w2[e].float().t()
         if b2 is not None:
             y = y + b2[e].float()
@@ -759,3 +763,127 @@ def row_norm(x, w, b, eps, kind):
     if b is not None:
         n = n + b.float()
     return n.to(w.dtype)
+
+
+def shift_norm(res, w, eps, x1, s1, x2, s2, w_offset, shift, state, seqs, out_dtype):
+    """``v = res + s1 x1 + s2 x2``; ``n = rmsnorm(v) (w_offset + w)``; with ``shift`` every row moves
+    towards the row before it, ``n[t] + (n[t-1] - n[t]) shift`` (the row before a sequence's first:
+    ``state[slot]``, zeros after a reset; the sequence's last n replaces it).  Returns (v, out)."""
+    v = res.float().clone()
+    if x1 is not None:
+        v += float(s1) * x1.float()
+    if x2 is not None:
+        v += float(s2) * x2.float()
+    n = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * (float(w_offset) + w.float())
+    if shift is None:
+        return v, n.to(out_dtype or w.dtype)
+    cu, slot, reset = seqs
+    out = torch.empty_like(n)
+    mu = shift.float()
+    for s in range(len(slot)):
+        r0, r1 = int(cu[s]), int(cu[s + 1])
+        if r1 <= r0:
+            continue
+        st = state[int(slot[s])]
+        prev = torch.cat([torch.zeros_like(n[:1]) if int(reset[s]) else st[None].float(), n[r0:r1 - 1]], 0)
+        out[r0:r1] = n[r0:r1] + (prev - n[r0:r1]) * mu
+        st.copy_(n[r1 - 1])
+    return v, out.to(out_dtype or w.dtype)
+
+
+def conv_rope_cache(q, k, v, wq, wk, wv, tail, seqs, positions, cos_sin, rot_dim, interleaved, unit_norm, eps, q_out,
+                    k_cache, v_cache, slots, Hq, Hkv, dim, vdim, P) -> None:
+    """Depthwise causal convolution of q / k / v over time (taps ``w*`` [C, K], no bias, no
+    activation; ``tail`` [slots, K-1, C] holds every sequence's last K-1 projected rows, C = all q,
+    k, v channels), rotary embedding of q and k, then (``unit_norm``) each head divided by its root
+    mean square, q -> ``q_out`` [T, Hq, D], k / v -> paged cache."""
+    T = q.shape[0]
+    if T == 0:
+        return
+    D = k_cache.shape[3]
+    x = torch.cat([q, k, v], 1).float()
+    if wq is not None:
+        wt = torch.cat([wq, wk, wv], 0).float()                    # [C, K]
+        K = wt.shape[1]
+        cu, slot, reset = seqs
+        y = torch.empty_like(x)
+        for s in range(len(slot)):
+            r0, r1 = int(cu[s]), int(cu[s + 1])
+            if r1 <= r0:
+                continue
+            if K > 1:
+                st = tail[int(slot[s])]
+                prev = torch.zeros_like(st).float() if int(reset[s]) else st.float()
+                seq = torch.cat([prev, x[r0:r1]], 0)               # [K-1+L, C]
+                st.copy_(seq[-(K - 1):].to(st.dtype))
+            else:
+                seq = x[r0:r1]
+            L = r1 - r0
+            y[r0:r1] = sum(wt[:, j] * seq[j:j + L] for j in range(K))
+        x = y
+    nq, nk = Hq * dim, Hkv * dim
+    half = rot_dim // 2
+    cs = cos_sin[positions.long()].float()
+    cos, sin = cs[:, None, :half], cs[:, None, half:rot_dim]
+
+    def prep(z, H):
+        z = z.reshape(T, H, dim).clone()
+        if rot_dim > 0:
+            if interleaved:
+                a, b = z[..., 0:rot_dim:2].clone(), z[..., 1:rot_dim:2].clone()
+                z[..., 0:rot_dim:2] = a * cos - b * sin
+                z[..., 1:rot_dim:2] = b * cos + a * sin
+            else:
+                a, b = z[..., :half].clone(), z[..., half:rot_dim].clone()
+                z[..., :half] = a * cos - b * sin
+                z[..., half:rot_dim] = b * cos + a * sin
+        if unit_norm:
+            z = z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps)
+        return z
+
+    qf, kf = prep(x[:, :nq], Hq), prep(x[:, nq:nq + nk], Hkv)
+    q_out.zero_()
+    q_out[:, :, :dim] = qf.to(q_out.dtype)
+    ok = slots >= 0
+    sl = slots[ok].long()
+    page, off = sl // P, sl % P
+    kp = torch.zeros(int(ok.sum()), Hkv, D, dtype=k_cache.dtype, device=k_cache.device)
+    kp[:, :, :dim] = kf[ok].to(k_cache.dtype)
+    vp = torch.zeros(int(ok.sum()), Hkv, D, dtype=v_cache.dtype, device=v_cache.device)
+    vp[:, :, :vdim] = x[:, nq + nk:].reshape(T, Hkv, vdim)[ok].to(v_cache.dtype)
+    k_cache[page, :, off, :] = kp
+    v_cache[page, :, :, off] = vp
+
+
+def talking_attn(q, k_cache, v_cache, block_tables, row_seq, row_pos, scale, window, sinks, r1, r2, talk, gate, vdim,
+                 out):
+    """Row t (block-table row ``row_seq[t]``, position ``row_pos[t]``, < 0: padding) attends keys
+    j in (pos - window, pos]: score q.k scale - r1 ln(1 + r2 (pos - j)), softmax whose denominator
+    also holds exp(sink), weights mixed over heads by ``talk`` [H, H], applied to the values of the
+    head's own kv head, times sigmoid(gate) per head."""
+    T, H, D = q.shape
+    Hkv, P = k_cache.shape[1], k_cache.shape[2]
+    G = H // Hkv
+    for t in range(T):
+        pos = int(row_pos[t])
+        if pos < 0:
+            out[t] = 0
+            continue
+        lo = max(0, pos - window + 1) if window > 0 else 0
+        keys = torch.arange(lo, pos + 1, device=q.device)
+        bt = block_tables[int(row_seq[t])]
+        pages, off = bt[(keys // P).long()].long(), keys % P
+        k = k_cache[pages, :, off, :].float()                      # [n, Hkv, D]
+        v = v_cache[pages, :, :, off].float()[:, :, :vdim]         # [n, Hkv, vdim]
+        s = torch.einsum("hd,nhd->hn", q[t].float(), k.repeat_interleave(G, 1)) * scale
+        s = s - r1.float()[:, None] * torch.log1p(r2.float()[:, None] * (pos - keys).float()[None])
+        if sinks is not None:
+            p = torch.softmax(torch.cat([s, sinks.float()[:, None]], 1), -1)[:, :-1]
+        else:
+            p = torch.softmax(s, -1)
+        p = talk.float() @ p
+        o = torch.einsum("hn,nhd->hd", p, v.repeat_interleave(G, 1))
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t].float())[:, None]
+        out[t] = o.reshape(-1).to(out.dtype)
+    return out
