@@ -612,11 +612,13 @@ OME_API int ome_conv_rope_cache(const void* q, int64_t q_stride, const void* k, 
   dim3 grid(Hq + 2 * Hkv, S, tiles);
 #define CRC_LAUNCH(TT)                                                                                              \
   do {                                                                                                              \
-    if (lds > 64 * 1024) {                                                                                          \
-      hipError_t e_ = hipFuncSetAttribute((const void*)conv_rope_cache_kernel<TT>,                                  \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                    \
-      if (e_ != hipSuccess) return (int)e_;                                                                         \
-    }                                                                                                               \
+    static bool big_ = false; /* once: allow the largest dynamic LDS block */                                       \
+    if (lds > 64 * 1024 && !big_) {                                                                                \
+      hipError_t e_ = hipFuncSetAttribute((const void*)conv_rope_cache_kernel<TT>,                                                \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                \
+      if (e_ != hipSuccess) return (int)e_;                                                                        \
+      big_ = true;                                                                                                 \
+    }                                                                                                              \
     conv_rope_cache_kernel<TT><<<grid, 256, lds, stream>>>(                                                         \
         (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, (const TT*)wq, (const TT*)wk,       \
         (const TT*)wv, K, (TT*)tail, cu, slot, reset, positions, cos_sin, rot_dim, interleaved, unit_norm, eps,     \

@@ -218,11 +218,13 @@ OME_API int ome_talking_attn(const void* q, int64_t q_stride, const void* k_cach
   const size_t lds = (size_t)(fixed + 2 * H * CH) * sizeof(float);
 #define TA_LAUNCH(TT)                                                                                                \
   do {                                                                                                               \
-    if (lds > 64 * 1024) {                                                                                           \
-      hipError_t e_ = hipFuncSetAttribute((const void*)talking_attn_kernel<TT>,                                      \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                     \
-      if (e_ != hipSuccess) return (int)e_;                                                                          \
-    }                                                                                                                \
+    static bool big_ = false; /* once: allow the largest dynamic LDS block */                                       \
+    if (lds > 64 * 1024 && !big_) {                                                                                \
+      hipError_t e_ = hipFuncSetAttribute((const void*)talking_attn_kernel<TT>,                                                \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                \
+      if (e_ != hipSuccess) return (int)e_;                                                                        \
+      big_ = true;                                                                                                 \
+    }                                                                                                              \
     talking_attn_kernel<TT><<<T, 256, lds, stream>>>(                                                                \
         (const TT*)q, q_stride, (const TT*)k_cache, (const TT*)v_cache, block_tables, bt_stride, row_seq, row_pos,   \
         (const TT*)gate, gate_stride, (TT*)out, out_stride, H, Hkv, D, vdim, P, scale, window, sinks, r1, r2, talk,  \
