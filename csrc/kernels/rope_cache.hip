@@ -468,12 +468,19 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
     T* __restrict__ tail, const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ reset,
     const int* __restrict__ positions, const float* __restrict__ cos_sin, int rot_dim, int interleaved,
     int unit_norm, float eps, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
-    const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P) {
+    const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P, int S) {
   extern __shared__ float sm[];   // [CR_TILE + K - 1][d] input rows, then [K][d] taps
-  const int hh = blockIdx.x, s = blockIdx.y;
+  const int hh = blockIdx.x;
+  // blockIdx.y counts the tiles of all sequences in turn (the grid is the upper bound T / CR_TILE + S)
+  int s = 0, z = blockIdx.y;
+  for (; s < S; ++s) {
+    const int n = (cu[s + 1] - cu[s] + CR_TILE - 1) / CR_TILE;
+    if (z < n) break;
+    z -= n;
+  }
+  if (s >= S) return;
   const int r0 = cu[s], r1 = cu[s + 1];
-  const int a = r0 + blockIdx.z * CR_TILE;
-  if (a >= r1) return;
+  const int a = r0 + z * CR_TILE;
   const int e = min(a + CR_TILE, r1);
   const int kind = hh < Hq ? 0 : (hh < Hq + Hkv ? 1 : 2);
   const int head = kind == 0 ? hh : (kind == 1 ? hh - Hq : hh - Hq - Hkv);
@@ -491,6 +498,20 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
   T* tl = KT > 0 ? tail + (int64_t)slot[s] * KT * C + c0 : nullptr;
   const bool fresh = reset[s] != 0;
   // input rows a - KT .. e - 1 of the sequence (before r0: the old tail, or zeros)
+  const bool vec = sizeof(T) == 2 && (d & 7) == 0 && (sstride & 7) == 0 && (C & 7) == 0 &&
+                   ((uintptr_t)src & 15) == 0 && (tl == nullptr || ((uintptr_t)tl & 15) == 0);
+  if (vec) {
+    const int cpr = d >> 3;   // 16-byte pieces per row
+    for (int i = tid; i < (e - a + KT) * cpr; i += 256) {
+      const int rr = i / cpr, c = (i - rr * cpr) << 3;
+      const int r = a - KT + rr;
+      bf16x8 x = {};
+      if (r >= r0) x = ld8((const bf16*)src + (int64_t)r * sstride + head * d + c);
+      else if (!fresh) x = ld8((const bf16*)tl + (int64_t)(KT + (r - r0)) * C + c);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) rows[rr * d + c + j] = (float)x[j];
+    }
+  } else
   for (int i = tid; i < (e - a + KT) * d; i += 256) {
     const int rr = i / d, c = i - rr * d;
     const int r = a - KT + rr;
@@ -500,7 +521,7 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
     rows[rr * d + c] = x;
   }
   __syncthreads();
-  if (blockIdx.z == 0 && KT > 0) {   // new tail: inputs L - KT .. L - 1 of the step; negative = old tail rows
+  if (z == 0 && KT > 0) {   // new tail: inputs L - KT .. L - 1 of the step; negative = old tail rows
     const int L = r1 - r0;
     for (int i = tid; i < KT * d; i += 256) {
       const int j = i / d, c = i - j * d;
@@ -604,12 +625,12 @@ OME_API int ome_conv_rope_cache(const void* q, int64_t q_stride, const void* k, 
   if (dim <= 0 || vdim <= 0 || dim > D || vdim > D || D > 256 || K < 0 || K > 33 || rot_dim > dim || (rot_dim & 1))
     return -2;
   if (K > 0 && (wq == nullptr || wk == nullptr || wv == nullptr || (K > 1 && tail == nullptr))) return -2;
-  const int tiles = (T + CR_TILE - 1) / CR_TILE;
-  if (tiles > 65535 || S > 65535) return -3;
+  const int tiles = (T + CR_TILE - 1) / CR_TILE + S;
+  if (tiles > 65535) return -3;
   const int dmax = dim > vdim ? dim : vdim;
   const size_t lds = (size_t)((CR_TILE + (K > 0 ? K - 1 : 0)) * dmax + K * dmax) * sizeof(float);
   if (lds > 160 * 1024) return -3;
-  dim3 grid(Hq + 2 * Hkv, S, tiles);
+  dim3 grid(Hq + 2 * Hkv, tiles);
 #define CRC_LAUNCH(TT)                                                                                              \
   do {                                                                                                              \
     static bool big_ = false; /* once: allow the largest dynamic LDS block */                                       \
@@ -622,7 +643,7 @@ OME_API int ome_conv_rope_cache(const void* q, int64_t q_stride, const void* k, 
     conv_rope_cache_kernel<TT><<<grid, 256, lds, stream>>>(                                                         \
         (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, (const TT*)wq, (const TT*)wk,       \
         (const TT*)wv, K, (TT*)tail, cu, slot, reset, positions, cos_sin, rot_dim, interleaved, unit_norm, eps,     \
-        (TT*)q_out, (TT*)k_cache, (TT*)v_cache, slots, Hq, Hkv, dim, vdim, D, P);                                   \
+        (TT*)q_out, (TT*)k_cache, (TT*)v_cache, slots, Hq, Hkv, dim, vdim, D, P, S);                                \
   } while (0)
   if (f32) CRC_LAUNCH(float);
   else CRC_LAUNCH(bf16);

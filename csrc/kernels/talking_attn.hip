@@ -236,3 +236,273 @@ OME_API int ome_talking_attn(const void* q, int64_t q_stride, const void* k_cach
   OME_CHECK_LAUNCH();
   return 0;
 }
+
+// ------------------------------------------------------------------------------------------
+// Prompt chunks on the matrix cores (bf16).  One workgroup = 16 consecutive query rows of one
+// sequence (a quarter / half of a prefill work item) x ALL heads; wave w owns heads w, w + NW, ...
+// (at most HPW of them, NW = waves of the workgroup).  Keys go by in tiles of 32 (two pages):
+//
+//   pass 1   per head: S^T = K Q^T (MFMA 16x16x32; lane (n, g) holds row n, keys 16X + 4g + i),
+//            bias, mask, running maximum and sum per row -> with the sink, m and 1 / l to LDS.
+//   pass 2   per key tile, all waves in step:
+//            (a) per head: S^T again, the FINAL weights p = exp2(s - m) / l as bf16 into
+//                Pb[column = (key slot, row)][head]          (head = the next product's k index)
+//            (b) the mix as a matrix product: P'[h, column] = sum_g talk[h, g] Pb[column, g]
+//                (MFMA, M = 16 heads h, K = 32 heads g, N = the 16 rows of one key slot), written as
+//                bf16 into Pm[head][row][key slot]
+//            (c) per head: O^T += V^T P'^T with the values of the head's own kv head (the key
+//                slots are in the order the value fragment cat(page A keys 4g.., page B keys 4g..)
+//                has them, so Pm rows are read as 16-byte B fragments).
+//
+// The weights are final before they are mixed, so the accumulator is never rescaled.  Scores,
+// maxima and sums are fp32 (log2 domain); weights enter the two products as bf16, like the weights
+// of every MFMA attention kernel here; talk is taken as bf16 (what a 16-bit checkpoint stores).
+// ------------------------------------------------------------------------------------------
+namespace {
+
+__device__ __forceinline__ f32x4 ta_mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ bf16x8 ta_cat44(bf16x4 a, bf16x4 b) {
+  return bf16x8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+}
+
+constexpr int TP_PAD = 8;   // bf16 elements of padding per LDS row
+
+template <int D, int HPW>
+__global__ __launch_bounds__(512) void talking_prefill_kernel(
+    const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu_q,
+    const int* __restrict__ kv_lens, const int2* __restrict__ items, const bf16* __restrict__ gate,
+    int64_t gate_stride, bf16* __restrict__ out, int64_t out_stride, int H, int Hkv, int vdim, float mul, int window,
+    const float* __restrict__ sinks, const float* __restrict__ r1, const float* __restrict__ r2,
+    const float* __restrict__ talk) {
+  constexpr int P = 16, NB = D / 16, KS = D / 32;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int HP = (H + 31) & ~31;          // heads as a k dimension
+  const int HM = (H + 15) & ~15;          // heads as an m dimension
+  const int ldb = HP + TP_PAD, ldm = 32 + TP_PAD;
+  bf16* Pb = reinterpret_cast<bf16*>(smem);              // [512][ldb]
+  bf16* Pm = Pb + 512 * ldb;                             // [H][16][ldm]
+  bf16* Tk = Pm + H * 16 * ldm;                          // [HM][ldb]
+  float* ml = reinterpret_cast<float*>(Tk + HM * ldb);   // [H][16][2]: m (log2 domain), 1 / l
+  const int2 it = items[blockIdx.x];
+  const int s = it.x, r0 = it.y + 16 * blockIdx.y;
+  const int q0 = cu_q[s];
+  const int q_len = cu_q[s + 1] - q0;
+  if (r0 >= q_len) return;
+  const int kv_len = kv_lens[s];
+  const int prefix = kv_len - q_len;
+  const int G = H / Hkv;
+  const int NW = blockDim.x >> 6;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int n = lane & 15, g = lane >> 4;
+  const int r_hi = min(r0 + 16, q_len);
+  const int kv_end = min(kv_len, prefix + r_hi);
+  const int lo0 = window > 0 ? max(0, prefix + r0 - window + 1) : 0;
+  const int kv_lo = lo0 & ~31;
+  const int* bt = block_tables + (int64_t)s * bt_stride;
+  const int64_t kpage = (int64_t)Hkv * P * D;
+  const int r = r0 + n;                       // this lane's query row
+  const bool row_ok = r < q_len;
+  const int qpos = prefix + r;
+  const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
+
+  for (int i = threadIdx.x; i < HM * ldb; i += blockDim.x) {   // talk as bf16, zero padded
+    const int h = i / ldb, c = i - h * ldb;
+    Tk[i] = (bf16)((h < H && c < H) ? talk[h * H + c] : 0.f);
+  }
+  for (int i = threadIdx.x; i < 512 * ldb; i += blockDim.x) Pb[i] = (bf16)0.f;   // (pad heads stay zero)
+
+  // ---- pass 1
+  for (int j = 0; j < HPW; ++j) {
+    const int head = wave + NW * j;
+    if (head >= H) break;
+    const int kvh = head / G;
+    bf16x8 qf[KS];
+    const bf16* qr = q + (int64_t)(q0 + min(r, q_len - 1)) * q_stride + (int64_t)head * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = ld8(qr + 32 * ks + 8 * g);
+    const float b1 = r1[head], b2 = r2[head];
+    float m_i = -__builtin_inff(), l_i = 0.f;
+    for (int kb = kv_lo; kb < kv_end; kb += 32) {
+      const int pA = bt[kb / P];
+      const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
+      const bf16* kA = k_cache + pA * kpage + (int64_t)kvh * P * D;
+      const bf16* kB = k_cache + pB * kpage + (int64_t)kvh * P * D;
+      f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        sc[0] = ta_mfma(ld8(kA + n * D + 32 * ks + 8 * g), qf[ks], sc[0]);
+        sc[1] = ta_mfma(ld8(kB + n * D + 32 * ks + 8 * g), qf[ks], sc[1]);
+      }
+      float mt = -__builtin_inff();
+#pragma unroll
+      for (int X = 0; X < 2; ++X)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 16 * X + 4 * g + i;
+          const bool ok = row_ok && key <= qpos && key >= lo;
+          const float v = ok ? sc[X][i] * mul - b1 * __log2f(1.f + b2 * (float)(qpos - key)) : -__builtin_inff();
+          sc[X][i] = v;
+          mt = fmaxf(mt, v);
+        }
+      mt = group4_max(mt);
+      const float m_new = fmaxf(m_i, mt);
+      const float m_use = (m_new == -__builtin_inff()) ? 0.f : m_new;
+      float rs = 0.f;
+#pragma unroll
+      for (int X = 0; X < 2; ++X)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rs += __builtin_amdgcn_exp2f(sc[X][i] - m_use);
+      rs = group4_sum(rs);
+      l_i = l_i * __builtin_amdgcn_exp2f(m_i - m_use) + rs;
+      m_i = m_new;
+    }
+    if (sinks != nullptr) {
+      const float sk = sinks[head] * 1.4426950408889634f;
+      const float m_new = fmaxf(m_i, sk);
+      l_i = l_i * __builtin_amdgcn_exp2f(m_i - m_new) + __builtin_amdgcn_exp2f(sk - m_new);
+      m_i = m_new;
+    }
+    if (g == 0) {
+      ml[(head * 16 + n) * 2] = (m_i == -__builtin_inff()) ? 0.f : m_i;
+      ml[(head * 16 + n) * 2 + 1] = l_i > 0.f ? 1.f / l_i : 0.f;
+    }
+  }
+  __syncthreads();
+
+  // ---- pass 2
+  f32x4 o[HPW][NB];
+#pragma unroll
+  for (int j = 0; j < HPW; ++j)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) o[j][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int kb = kv_lo; kb < kv_end; kb += 32) {
+    const int pA = bt[kb / P];
+    const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
+    // (a) final weights of this wave's heads
+    for (int j = 0; j < HPW; ++j) {
+      const int head = wave + NW * j;
+      if (head >= H) break;
+      const int kvh = head / G;
+      const bf16* qr = q + (int64_t)(q0 + min(r, q_len - 1)) * q_stride + (int64_t)head * D;
+      const bf16* kA = k_cache + pA * kpage + (int64_t)kvh * P * D;
+      const bf16* kB = k_cache + pB * kpage + (int64_t)kvh * P * D;
+      f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8 qv = ld8(qr + 32 * ks + 8 * g);
+        sc[0] = ta_mfma(ld8(kA + n * D + 32 * ks + 8 * g), qv, sc[0]);
+        sc[1] = ta_mfma(ld8(kB + n * D + 32 * ks + 8 * g), qv, sc[1]);
+      }
+      const float b1 = r1[head], b2 = r2[head];
+      const float m = ml[(head * 16 + n) * 2], il = ml[(head * 16 + n) * 2 + 1];
+#pragma unroll
+      for (int X = 0; X < 2; ++X)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + 16 * X + 4 * g + i;
+          const bool ok = row_ok && key <= qpos && key >= lo;
+          const float v = sc[X][i] * mul - b1 * __log2f(1.f + b2 * (float)(qpos - key));
+          const float p = ok ? __builtin_amdgcn_exp2f(v - m) * il : 0.f;
+          Pb[((8 * g + 4 * X + i) * 16 + n) * ldb + head] = (bf16)p;
+        }
+    }
+    __syncthreads();
+    // (b) mix over heads: one key slot (16 rows) per product column block
+    for (int t = wave; t < 32; t += NW) {
+      for (int mt = 0; mt < HM / 16; ++mt) {
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int ks = 0; ks < HP / 32; ++ks)
+          acc = ta_mfma(*reinterpret_cast<const bf16x8*>(Tk + (16 * mt + n) * ldb + 32 * ks + 8 * g),
+                        *reinterpret_cast<const bf16x8*>(Pb + (16 * t + n) * ldb + 32 * ks + 8 * g), acc);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int h = 16 * mt + 4 * g + i;
+          if (h < H) Pm[(h * 16 + n) * ldm + t] = (bf16)acc[i];
+        }
+      }
+    }
+    __syncthreads();
+    // (c) values
+    for (int j = 0; j < HPW; ++j) {
+      const int head = wave + NW * j;
+      if (head >= H) break;
+      const int kvh = head / G;
+      const bf16* vA = v_cache + pA * kpage + (int64_t)kvh * D * P;
+      const bf16* vB = v_cache + pB * kpage + (int64_t)kvh * D * P;
+      const bf16x8 pb = *reinterpret_cast<const bf16x8*>(Pm + (head * 16 + n) * ldm + 8 * g);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const int dim = 16 * nb + n;
+        o[j][nb] = ta_mfma(ta_cat44(ld4(vA + dim * P + 4 * g), ld4(vB + dim * P + 4 * g)), pb, o[j][nb]);
+      }
+    }
+    // (the next tile's (a) writes Pb only, and its (b) follows a barrier after this tile's (c))
+  }
+  // ---- epilogue: O^T lane (row n, dims 16 nb + 4 g + i), times the head's gate
+  if (row_ok) {
+#pragma unroll
+    for (int j = 0; j < HPW; ++j) {
+      const int head = wave + NW * j;
+      if (head < H) {
+        const float gt = gate != nullptr
+                             ? 1.f / (1.f + __expf(-(float)gate[(int64_t)(q0 + r) * gate_stride + head])) : 1.f;
+        bf16* orow = out + (int64_t)(q0 + r) * out_stride + (int64_t)head * vdim;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int dim = 16 * nb + 4 * g + i;
+            if (dim < vdim) orow[dim] = (bf16)(o[j][nb][i] * gt);
+          }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+// items int32 [n_items, 2] = (sequence, first row) of `item_rows`-row work items (a multiple of 16);
+// sequence s owns query rows cu_q[s] .. cu_q[s + 1] at positions kv_lens[s] - q_len ...; bf16 only.
+OME_API int ome_talking_prefill(const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                                const int* block_tables, int bt_stride, const int* cu_q, const int* kv_lens,
+                                const int* items, int n_items, int item_rows, const void* gate, int64_t gate_stride,
+                                void* out, int64_t out_stride, int H, int Hkv, int D, int vdim, int P, float scale,
+                                int window, const float* sinks, const float* r1, const float* r2, const float* talk,
+                                hipStream_t stream) {
+  if (n_items <= 0) return 0;
+  if (P != 16 || H <= 0 || Hkv <= 0 || H % Hkv || vdim <= 0 || vdim > D || item_rows <= 0 || item_rows % 16 ||
+      (q_stride & 7) || r1 == nullptr || r2 == nullptr || talk == nullptr)
+    return -2;
+  const int hpw = D == 256 ? 2 : 4;
+  const int NW = (H + hpw - 1) / hpw;
+  if (NW > 8) return -3;   // (8 waves: the accumulators of HPW heads fit the registers of 2 waves per SIMD)
+  const int HP = (H + 31) & ~31, HM = (H + 15) & ~15, ldb = HP + TP_PAD, ldm = 32 + TP_PAD;
+  const size_t lds = (size_t)(512 * ldb + H * 16 * ldm + HM * ldb) * 2 + (size_t)H * 16 * 2 * 4;
+  if (lds > 160 * 1024) return -3;
+  const dim3 grid(n_items, item_rows / 16);
+  const float mul = scale * 1.4426950408889634f;
+#define TP_LAUNCH(DD, HH)                                                                                            \
+  do {                                                                                                               \
+    static bool big_ = false;                                                                                        \
+    if (lds > 64 * 1024 && !big_) {                                                                                  \
+      hipError_t e_ = hipFuncSetAttribute((const void*)talking_prefill_kernel<DD, HH>,                               \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                   \
+      if (e_ != hipSuccess) return (int)e_;                                                                          \
+      big_ = true;                                                                                                   \
+    }                                                                                                                \
+    talking_prefill_kernel<DD, HH><<<grid, 64 * NW, lds, stream>>>(                                                  \
+        (const bf16*)q, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, bt_stride, cu_q, kv_lens, \
+        (const int2*)items, (const bf16*)gate, gate_stride, (bf16*)out, out_stride, H, Hkv, vdim, mul, window, sinks, \
+        r1, r2, talk);                                                                                               \
+  } while (0)
+  if (D == 64) TP_LAUNCH(64, 4);
+  else if (D == 128) TP_LAUNCH(128, 4);
+  else if (D == 256) TP_LAUNCH(256, 2);
+  else return -2;
+#undef TP_LAUNCH
+  OME_CHECK_LAUNCH();
+  return 0;
+}

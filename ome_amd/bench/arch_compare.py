@@ -1,5 +1,11 @@
 """Layer-list designs beside their closest existing model at equal size (``bench.py --arch-compare
-[--arch-design zavilorn|metitar]``).
+[--arch-design zavilorn|metitar|milenex]``).
+
+Milenex (token shift, sliding-window attention with sinks: one kind with short convolutions, rotary
+pairs and unit-RMS q / k, one with a logarithmic distance bias and weights mixed across heads;
+group-routed clamped-GLU experts plus a gated shared expert) stands beside a GPT-OSS-style stack
+(sliding-window attention with sinks, clamped-GLU experts) of the same width, depth, heads, window
+and expert sizes.
 
 Metitar (latent attention + HGRN2, PolyNorm / input-scaled MoE feed-forwards) stands beside a
 DeepSeek-V2-style stack (multi-head latent attention, dense then routed feed-forwards with shared
@@ -92,6 +98,34 @@ def deepseek_like_config(s: dict) -> dict:
                 routed_scaling_factor=1.0, kv_lora_rank=256, q_lora_rank=s["q_rank"], qk_nope_head_dim=128,
                 qk_rope_head_dim=32, v_head_dim=128, vocab_size=s["vocab"], rms_norm_eps=1e-6, rope_theta=10000.0,
                 max_position_embeddings=8192, tie_word_embeddings=False)
+
+
+X_SIZES = {
+    "2k": dict(width=2048, heads=16, kv=4, experts=32, top=4, eff=1024, vocab=32768),
+    "4k": dict(width=4096, heads=32, kv=8, experts=32, top=4, eff=2048, vocab=32768),
+}
+
+
+def milenex_config(s: dict, window: int = 1024) -> dict:
+    """[talking-heads attention, conv + rotary attention] x 4, 128-wide heads, every layer with 32
+    experts in 4 groups (2 kept), top 4, and a gated shared expert of an expert's width."""
+    base = {"heads": s["heads"], "kv_heads": s["kv"], "dim": 128, "vdim": 128, "mask": {"size": window},
+            "scale": 128 ** -0.5}
+    rot = dict(base, conv=4, rot={"base": 10000.0, "dims": 64})
+    moe = {"kind": "moe", "router": {"experts": s["experts"], "top": s["top"], "groups": {"count": 4, "keep": 2}},
+           "expert": {"ff": s["eff"], "limit": 7.0}, "shared": {"ff": s["eff"], "limit": 7.0}}
+    layers = [{"type": "attention_2", "mixer": dict(base), "mlp": moe}, {"type": "attention", "mixer": rot, "mlp": moe}] * 4
+    return {"architecture": "Milenex", "layers": layers, "norm": {"eps": 1e-6}, "vocab": s["vocab"],
+            "width": s["width"], "max_positions": 8192}
+
+
+def gpt_oss_like_config(s: dict, window: int = 1024) -> dict:
+    """Eight sliding-window layers with sinks and clamped-GLU experts of the Milenex stack's sizes."""
+    return dict(architectures=["GptOssForCausalLM"], model_type="gpt_oss", hidden_size=s["width"],
+                num_hidden_layers=8, num_attention_heads=s["heads"], num_key_value_heads=s["kv"], head_dim=128,
+                intermediate_size=s["eff"], num_local_experts=s["experts"], num_experts_per_tok=s["top"],
+                vocab_size=s["vocab"], rms_norm_eps=1e-6, sliding_window=window, layer_types=["sliding_attention"] * 8,
+                attention_bias=True, max_position_embeddings=8192, rope_theta=10000.0, tie_word_embeddings=False)
 
 
 def _engine(name: str, cfg: dict, max_running: int, context: int):
@@ -364,8 +398,130 @@ def kernel_table_metitar(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
     return rows
 
 
+def kernel_table_milenex(T: int = 4096, B: int = 64, ctx: int = 4096, width: int = 4096) -> list[dict]:
+    """Milenex's kernels beside their like kernels (same columns as :func:`kernel_table`)."""
+    from ome_amd import ops
+    from ome_amd.models.config import plain_rope_table
+    from ome_amd.models.mixers import GroupRoutedMoE
+
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def pair(name, new, like, bytes_new, bytes_like, note="", iters=30):
+        tn, tl = _time_us(new, iters), _time_us(like, iters)
+        fn, fl = bytes_new / tn / 1e3 / HBM_GBS, bytes_like / tl / 1e3 / HBM_GBS
+        rows.append({"kernel": name, "us": round(tn, 1), "roofline": round(fn, 3), "like_us": round(tl, 1),
+                     "like_roofline": round(fl, 3), "vs_like": round(fl / max(fn, 1e-9), 2), "note": note})
+
+    def seqs(lens):
+        cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+        n = len(lens)
+        return cu, torch.arange(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev)
+
+    torch.manual_seed(0)
+    Hq, Hkv, D, P, W = 32, 8, 128, 16, 1024
+    for R, tag, lens in ((T, "prefill", [T // 8] * 8), (B, "decode", [1] * B)):
+        sq = seqs(lens)
+        # ---- stream update + offset norm (+ token shift) vs add + RMSNorm on a bf16 stream
+        res = torch.randn(R, width, device=dev)
+        y = torch.randn(R, width, device=dev).to(bf)
+        w, mu = torch.zeros(width, device=dev, dtype=bf), torch.rand(width, device=dev).to(bf)
+        st = torch.zeros(len(lens), width, device=dev)
+        rb, xb = res.to(bf), y.clone()
+        pair(f"shift_norm with token shift ({tag})",
+             lambda: ops.shift_norm(res, w, 1e-6, y, 1.0, None, 1.0, 1.0, mu, st, sq, bf),
+             lambda: ops.fused_add_rmsnorm(xb, rb, w, 1e-6), R * width * 12, R * width * 8,
+             "fp32 stream in and out of place: 12 B / element against 8; the row before is read again from cache")
+        pair(f"shift_norm, no shift ({tag})", lambda: ops.shift_norm(res, w, 1e-6, y, w_offset=1.0, out_dtype=bf),
+             lambda: ops.fused_add_rmsnorm(xb, rb, w, 1e-6), R * width * 12, R * width * 8)
+        # ---- convolution + rotary + unit norm + paged write vs per-head norm + rotary + paged write
+        n_pages = R // P + 2
+        kc = torch.zeros(n_pages, Hkv, P, D, device=dev, dtype=bf)
+        vc = torch.zeros(n_pages, Hkv, D, P, device=dev, dtype=bf)
+        C = (Hq + 2 * Hkv) * D
+        qkv = torch.randn(R, C, device=dev).to(bf)
+        pos = torch.arange(R, dtype=torch.int32, device=dev) % 2048
+        slots = torch.arange(R, dtype=torch.int32, device=dev) + P
+        cs = plain_rope_table(10000.0, 64, 2049, dev)
+        qo = torch.empty(R, Hq, D, device=dev, dtype=bf)
+        cw = [(torch.randn(c, 4, device=dev) * 0.3).to(bf) for c in (Hq * D, Hkv * D, Hkv * D)]
+        tail = torch.zeros(len(lens), 3, C, device=dev, dtype=bf)
+        hn = torch.ones(D, device=dev, dtype=bf)
+        nb = R * C * 2 * 2
+        pair(f"conv_rope_cache 4 taps ({tag})",
+             lambda: ops.conv_rope_cache(qkv[:, :Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D:], *cw, tail,
+                                         sq, pos, cs, 64, True, True, 1e-6, qo, kc, vc, slots, Hq, Hkv, D, D),
+             lambda: ops.rope_qkv_cache(qkv, pos, cs, 64, qo, kc, vc, slots, Hq, Hkv, D, True, hn, hn, 1e-6), nb, nb,
+             "like: Qwen3's per-head norm + rotary + cache write (no convolution)")
+        # ---- clamped GLU with the shared expert's per-row gate vs without
+        I = 2048
+        gu = torch.randn(R, 2 * I, device=dev).to(bf)
+        rg = torch.randn(R, 33, device=dev)
+        pair(f"act_and_mul row gate ({tag})", lambda: ops.act_and_mul(gu, 2, limit=7.0, row_gate=rg[:, 32]),
+             lambda: ops.act_and_mul(gu, 2), R * I * 6, R * I * 6)
+        # ---- routed feed-forward: grouped routing + gated shared expert vs GPT-OSS's experts
+        E, k, ff = 32, 4, 2048
+        moe = GroupRoutedMoE(width, E, k, ff, 7.0, 4, 2, ff, 7.0, dev, bf)
+        moe.init_random(torch.Generator(device=dev).manual_seed(1), 0.02)
+        x = torch.randn(R, width, device=dev).to(bf)
+        lg = torch.randn(R, E, device=dev)
+        tw, tid = ops.moe_route(lg, k, True, "softmax")
+        touched = min(E, R * k) * 3 * ff * width * 2
+        pair(f"group-routed moe 32 experts top 4 + shared ({tag})", lambda: moe.forward(x),
+             lambda: ops.fused_moe(x, tw, tid, moe.w13, moe.w2, 2, 1.0), touched + 3 * ff * width * 2, touched,
+             "new: router GEMM + route + shared expert (3 GEMMs) + grouped GEMMs + combine; like: grouped GEMMs + combine",
+             10)
+    # ---- attention with mixed heads: decode over a long context vs the sliding-window decode kernel with sinks
+    per = ctx // P
+    kc = (torch.randn(B * per + 1, Hkv, P, D, device=dev) * 0.3).to(bf)
+    vc = (torch.randn(B * per + 1, Hkv, D, P, device=dev) * 0.3).to(bf)
+    bt = (torch.arange(B * per, dtype=torch.int32, device=dev) + 1).view(B, per)
+    sl = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    q = (torch.randn(B, Hq, D, device=dev) * 0.3).to(bf)
+    gate = torch.randn(B, Hq, device=dev).to(bf)
+    sinks = torch.zeros(Hq, device=dev)
+    r1, r2 = torch.full((Hq,), 0.3, device=dev), torch.full((Hq,), 1.0, device=dev)
+    talk = torch.eye(Hq, device=dev) + 0.05
+    ws = ops.DecodeWorkspace(B, Hq, D, ctx, 0, dev, parts=4)
+    rows_i = torch.arange(B, dtype=torch.int32, device=dev)
+    kvb = B * Hkv * D * 2 * 2 * W
+    pair("talking_attn decode 64 x 4096 ctx, window 1024",
+         lambda: ops.talking_attn(q, kc, vc, bt, rows_i, sl - 1, 0.09, W, sinks, r1, r2, talk, gate, D),
+         lambda: ops.paged_decode(q, kc, vc, bt, sl, 0.09, ws, W, sinks=sinks), kvb, kvb,
+         "all heads of a row in one workgroup (the mix needs every head's final weight)", 10)
+    # ---- prefill, 2 x 2048 rows
+    q_lens = [2048, 2048]
+    Tq = sum(q_lens)
+    qp = (torch.randn(Tq, Hq, D, device=dev) * 0.3).to(bf)
+    gp = torch.randn(Tq, Hq, device=dev).to(bf)
+    cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device=dev)
+    kl = torch.tensor(q_lens, dtype=torch.int32, device=dev)
+    bt2 = (torch.arange(2 * 128, dtype=torch.int32, device=dev) + 1).view(2, 128)
+    items = torch.tensor(ops.prefill_work_items(q_lens, q_lens), dtype=torch.int32, device=dev)
+    tok_row = torch.arange(Tq, dtype=torch.int32, device=dev) // 2048
+    tok_pos = (torch.arange(Tq, dtype=torch.int32, device=dev) % 2048).to(torch.int32)
+    flops = 4.0 * Hq * D * sum(min(W, i + 1) for i in range(2048)) * 2
+    tn = _time_us(lambda: ops.talking_attn(qp, kc, vc, bt2, tok_row, tok_pos, 0.09, W, sinks, r1, r2, talk, gp, D), 5)
+    tl = _time_us(lambda: ops.paged_prefill(qp, kc, vc, bt2, cu, kl, items, 0.09, W, sinks=sinks), 5)
+    rows.append({"kernel": "talking_attn prefill 2 x 2048 rows, window 1024", "us": round(tn, 1),
+                 "roofline": round(flops / tn / 1e6 / 2.5e3, 3), "like_us": round(tl, 1),
+                 "like_roofline": round(flops / tl / 1e6 / 2.5e3, 3), "vs_like": round(tn / tl, 2),
+                 "note": "share of 2.5 PFLOP/s bf16 (q.k and p.v only); like: the MFMA sliding-window kernel with sinks"})
+    return rows
+
+
 def run(sizes=("2k", "4k"), kernels: bool = True, only: str | None = None, design: str = "zavilorn") -> dict:
     out = {"throughput": [], "kernels": []}
+    if design == "milenex":
+        for k in sizes:
+            s = X_SIZES[k]
+            if only in (None, "milenex"):
+                out["throughput"].append(throughput(f"milenex-{k}", milenex_config(s)))
+            if only in (None, "gpt-oss"):
+                out["throughput"].append(throughput(f"gpt-oss-like-{k}", gpt_oss_like_config(s)))
+        if kernels:
+            out["kernels"] = kernel_table_milenex()
+        return out
     if design == "metitar":
         for k in sizes:
             s = M_SIZES[k]
@@ -393,9 +549,9 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--sizes", default="2k,4k")
     ap.add_argument("--no-kernels", action="store_true")
-    ap.add_argument("--only", choices=["zavilorn", "nemotron", "metitar", "deepseek"], default=None,
+    ap.add_argument("--only", choices=["zavilorn", "nemotron", "metitar", "deepseek", "milenex", "gpt-oss"], default=None,
                     help="one stack (for kernel traces)")
-    ap.add_argument("--design", choices=["zavilorn", "metitar"], default="zavilorn")
+    ap.add_argument("--design", choices=["zavilorn", "metitar", "milenex"], default="zavilorn")
     ap.add_argument("--no-throughput", action="store_true", help="the kernel table only")
     a = ap.parse_args(argv)
     res = run(() if a.no_throughput else tuple(a.sizes.split(",")), not a.no_kernels, a.only, a.design)

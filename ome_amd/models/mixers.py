@@ -642,9 +642,19 @@ class TalkingHeadsAttention(_Block):
                                  self.Hkv, self.dim, self.vdim)
         o = torch.empty(T, self.Hq * self.vdim, dtype=h.dtype, device=h.device)
         gate = p[:, nq + nk + nv:]
-        for s, e, bt, rows, pos in attention_rows(ctx.meta, T):
-            ops.talking_attn(q[s:e], k_cache, v_cache, bt, rows, pos, self.scale, self.window, self.sink, self.r1,
-                             self.r2, self.talk, gate[s:e], self.vdim, out=o[s:e])
+        meta = ctx.meta
+        n = 0 if meta.is_decode else (meta.num_prefill if meta.mode == "mixed" else T)
+        if n and ops.talking_prefill_ok(q, self.Hq, self.D, k_cache.shape[2]):   # prompt chunks: the MFMA kernel
+            ops.talking_prefill(q[:n], k_cache, v_cache, meta.block_tables, meta.cu_q, meta.kv_lens, meta.items,
+                                self.scale, self.window, self.sink, self.r1, self.r2, self.talk, gate[:n], self.vdim,
+                                out=o[:n])
+        else:
+            n = 0
+        if n < T:                              # single rows (and every row of fp32 models): the row kernel
+            for s, e, bt, rows, pos in attention_rows(meta, T):
+                if e > n:
+                    ops.talking_attn(q[s:e], k_cache, v_cache, bt, rows, pos, self.scale, self.window, self.sink,
+                                     self.r1, self.r2, self.talk, gate[s:e], self.vdim, out=o[s:e])
         return linear(o, self.w_o)
 
 

@@ -2012,3 +2012,43 @@ def talking_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
          out.stride(0), T, H, Hkv, D, vdim, P, float(scale), int(window), _sinks(sinks), r1.data_ptr(), r2.data_ptr(),
          talk.data_ptr(), f32, stream_ptr())
     return out
+
+
+def talking_prefill_ok(q: torch.Tensor, H: int, D: int, P: int) -> bool:
+    """Can :func:`talking_prefill` run its matrix-core kernel (bf16 on the GPU, 16-token pages, a
+    64 / 128 / 256-wide tile, at most 8 waves of 4 heads -- 2 heads at 256)?"""
+    return bool(q.is_cuda and q.dtype == torch.bfloat16 and P == 16 and D in (64, 128, 256) and
+                H <= (16 if D == 256 else 32))
+
+
+def talking_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                    cu_q: torch.Tensor, kv_lens: torch.Tensor, items, scale: float, window: int,
+                    sinks: torch.Tensor | None, r1: torch.Tensor, r2: torch.Tensor, talk: torch.Tensor,
+                    gate: torch.Tensor | None, vdim: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """:func:`talking_attn` for prompt chunks described like :func:`paged_prefill`'s (sequence s owns
+    query rows ``cu_q[s]:cu_q[s+1]`` at positions ``kv_lens[s] - q_len ..``; ``items`` from
+    :func:`prefill_plan` / :func:`prefill_work_items`).  bf16 on the GPU with a shape of
+    :func:`talking_prefill_ok`: the MFMA kernel (16 rows x all heads per workgroup, two passes over
+    the keys, the mix over heads as a matrix product through LDS); anything else: the row kernel."""
+    T, H, D = q.shape
+    Hkv, P = k_cache.shape[1], k_cache.shape[2]
+    out = torch.empty(T, H * vdim, dtype=q.dtype, device=q.device) if out is None else out
+    if not talking_prefill_ok(q, H, D, P):
+        r = torch.arange(T, dtype=torch.int64, device=q.device)
+        seq = torch.bucketize(r, _i32(cu_q)[1:].long(), right=True).clamp_(max=cu_q.shape[0] - 2)
+        pos = _i32(kv_lens)[seq] - cu_q[seq + 1] + r
+        return talking_attn(q, k_cache, v_cache, block_tables, seq.to(torch.int32), pos.to(torch.int32), scale, window,
+                            sinks, r1, r2, talk, gate, vdim, out)
+    rows = 32
+    if isinstance(items, PrefillPlan):
+        rows, items = items.rows, items.items
+    assert q.stride(2) == 1 and q.stride(1) == D and k_cache.shape[3] == D and out.stride(1) == 1
+    assert gate is None or (gate.stride(1) == 1 and gate.dtype == q.dtype)
+    for t in (r1, r2, talk):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    call("ome_talking_prefill", q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+         _i32(block_tables).data_ptr(), block_tables.stride(0), _i32(cu_q).data_ptr(), _i32(kv_lens).data_ptr(),
+         _i32(items).data_ptr(), items.shape[0], int(rows), ptr(gate), gate.stride(0) if gate is not None else 0,
+         out.data_ptr(), out.stride(0), H, Hkv, D, vdim, P, float(scale), int(window), _sinks(sinks), r1.data_ptr(),
+         r2.data_ptr(), talk.data_ptr(), stream_ptr())
+    return out

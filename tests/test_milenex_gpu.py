@@ -115,6 +115,47 @@ def test_talking_attn_kernel(dt, H, Hkv, D, vdim, window, ctx):
     _close(got, want, dt, want.float().abs().max().item())
 
 
+@pytest.mark.parametrize("H,Hkv,D,vdim,window", [(6, 3, 64, 64, 9), (4, 1, 64, 7, 6), (32, 8, 128, 128, 100),
+                                                 (16, 2, 256, 200, 0), (1, 1, 64, 64, 40), (18, 9, 64, 2, 20),
+                                                 (12, 4, 128, 96, 33)])
+def test_talking_prefill_kernel(H, Hkv, D, vdim, window):
+    """Prompt chunks on the matrix-core kernel (fresh prompts, a chunk behind a prefix that crosses
+    the window, a single row, row counts that do not fill a tile) against the row reference."""
+    g = torch.Generator().manual_seed(H + D)
+    P = 16
+    q_lens, kv_lens = [37, 1, 50, 16], [37, 20, 150, 48]
+    n_pages = [-(-k // P) for k in kv_lens]
+    perm = (torch.randperm(sum(n_pages), generator=g) + 1).to(torch.int32)
+    bt = torch.zeros(len(q_lens), max(n_pages), dtype=torch.int32)
+    a = 0
+    for s, n in enumerate(n_pages):
+        bt[s, :n] = perm[a:a + n]
+        a += n
+    kc = (torch.randn(sum(n_pages) + 2, Hkv, P, D, generator=g) * 0.5).to(BF)
+    vc = torch.randn(sum(n_pages) + 2, Hkv, D, P, generator=g).to(BF)
+    T = sum(q_lens)
+    q = (torch.randn(T, H, D, generator=g) * 0.5).to(BF)
+    gate = torch.randn(T, H + 5, generator=g).to(BF)
+    r1, r2 = torch.rand(H, generator=g), torch.rand(H, generator=g) * 2 + 0.1
+    talk = (torch.eye(H) + torch.randn(H, H, generator=g) * 0.3).to(BF).float()
+    sinks = torch.randn(H, generator=g)
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    kl = torch.tensor(kv_lens, dtype=torch.int32)
+    seq = torch.cat([torch.full((n,), s) for s, n in enumerate(q_lens)]).to(torch.int32)
+    pos = torch.cat([torch.arange(k - n, k) for n, k in zip(q_lens, kv_lens)]).to(torch.int32)
+    want = ops.talking_attn(q, kc, vc, bt, seq, pos, 0.2, window, sinks, r1, r2, talk, gate[:, :H], vdim)
+    items = torch.tensor(ops.prefill_work_items(q_lens, kv_lens), dtype=torch.int32, device=DEV)
+    d = lambda t: t.to(DEV)   # noqa: E731
+    assert ops.talking_prefill_ok(d(q), H, D, P)
+    got = ops.talking_prefill(d(q), d(kc), d(vc), d(bt), d(cu), d(kl), items, 0.2, window, d(sinks), d(r1), d(r2),
+                              d(talk), d(gate)[:, :H], vdim)
+    _close(got, want, BF, want.float().abs().max().item())
+    got = ops.talking_prefill(d(q), d(kc), d(vc), d(bt), d(cu), d(kl), items, 0.2, window, None, d(r1), d(r2), d(talk),
+                              None, vdim)
+    want = ops.talking_attn(q, kc, vc, bt, seq, pos, 0.2, window, None, r1, r2, talk, None, vdim)
+    _close(got, want, BF, want.float().abs().max().item())
+
+
 @pytest.mark.parametrize("dt", DTYPES)
 def test_small_ops(dt):
     g = torch.Generator().manual_seed(2)
