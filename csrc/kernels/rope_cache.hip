@@ -460,6 +460,7 @@ OME_API int ome_wide_norm_rope_cache(const void* q, int64_t q_stride, const void
 // ------------------------------------------------------------------------------------------
 namespace {
 constexpr int CR_TILE = 32;
+constexpr int CR_MAXS = 1024;   // sequence starts staged in LDS (more: read from global memory)
 
 template <typename T>
 __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
@@ -471,10 +472,18 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
     const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P, int S) {
   extern __shared__ float sm[];   // [CR_TILE + K - 1][d] input rows, then [K][d] taps
   const int hh = blockIdx.x;
-  // blockIdx.y counts the tiles of all sequences in turn (the grid is the upper bound T / CR_TILE + S)
+  // blockIdx.y counts the tiles of all sequences in turn (the grid is the upper bound T / CR_TILE + S);
+  // the sequence starts are staged in LDS so that the walk is not a chain of global loads
+  __shared__ int s_cu[CR_MAXS + 1];
+  const bool staged = S <= CR_MAXS;
+  if (staged) {
+    for (int i = threadIdx.x; i <= S; i += 256) s_cu[i] = cu[i];
+    __syncthreads();
+  }
+  const int* cus = staged ? s_cu : cu;
   int s = 0, z = blockIdx.y;
   for (; s < S; ++s) {
-    const int n = (cu[s + 1] - cu[s] + CR_TILE - 1) / CR_TILE;
+    const int n = (cus[s + 1] - cus[s] + CR_TILE - 1) / CR_TILE;
     if (z < n) break;
     z -= n;
   }
@@ -531,12 +540,14 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
   }
   const int wave = tid >> 6, lane = tid & 63;
   const int half = rot_dim >> 1;
+  // a lane owns two pairs of neighbouring channels: register u <-> channel (u >> 1) * 128 + 2 lane + (u & 1)
+  // (d <= 256), so an interleaved rotary pair sits in one lane and stores are 4 bytes wide
   for (int r = a + wave; r < e; r += 4) {
     const int rr = r - a;   // output row rr reads input rows rr .. rr + KT
-    float y[4];             // channels lane, lane + 64, lane + 128, lane + 192 (d <= 256)
+    float y[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int c = lane + 64 * u;
+      const int c = (u >> 1) * 128 + 2 * lane + (u & 1);
       float acc = 0.f;
       if (c < d) {
         if (K > 0)
@@ -551,8 +562,10 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
       if (slot_t >= 0) {
         T* vc = v_cache + (((int64_t)(slot_t / P) * Hkv + head) * D) * P + slot_t % P;
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (lane + 64 * u < d) vc[(int64_t)(lane + 64 * u) * P] = (T)y[u];
+        for (int u = 0; u < 4; ++u) {
+          const int c = (u >> 1) * 128 + 2 * lane + (u & 1);
+          if (c < d) vc[(int64_t)c * P] = (T)y[u];
+        }
       }
       continue;
     }
@@ -560,31 +573,34 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
       const float* cs = cos_sin + (int64_t)positions[r] * rot_dim;
       if (interleaved) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int c = lane + 64 * u;
-          const float other = __shfl_xor(y[u], 1);
+        for (int u = 0; u < 4; u += 2) {
+          const int c = (u >> 1) * 128 + 2 * lane;
           if (c < rot_dim) {
             const float co = cs[c >> 1], si = cs[half + (c >> 1)];
-            y[u] = (c & 1) ? y[u] * co + other * si : y[u] * co - other * si;
+            const float ev = y[u], od = y[u + 1];
+            y[u] = ev * co - od * si;
+            y[u + 1] = od * co + ev * si;
           }
         }
-      } else {   // channel i pairs with i + half: the partner sits in lane pc & 63, register pc >> 6
+      } else {   // channel i pairs with i + half: the partner pc sits in lane (pc & 127) >> 1, register
+        // (pc >> 7) * 2 + (pc & 1)
         float other[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          const int c = lane + 64 * u;
+          const int c = (u >> 1) * 128 + 2 * lane + (u & 1);
           const int pc = c < half ? c + half : c - half;
+          const int pl = (pc & 127) >> 1, pr = ((pc >> 7) << 1) | (pc & 1);
           float o = 0.f;
 #pragma unroll
           for (int u2 = 0; u2 < 4; ++u2) {
-            const float cand = __shfl(y[u2], pc & 63);
-            if ((pc >> 6) == u2) o = cand;
+            const float cand = __shfl(y[u2], pl);
+            if (pr == u2) o = cand;
           }
           other[u] = o;
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-          const int c = lane + 64 * u;
+          const int c = (u >> 1) * 128 + 2 * lane + (u & 1);
           if (c < rot_dim) {
             const int i = c < half ? c : c - half;
             const float co = cs[i], si = cs[half + i];
@@ -596,7 +612,7 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
     if (unit_norm) {
       float ss = 0.f;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) ss += (lane + 64 * u < d) ? y[u] * y[u] : 0.f;
+      for (int u = 0; u < 4; ++u) ss += ((u >> 1) * 128 + 2 * lane + (u & 1) < d) ? y[u] * y[u] : 0.f;
       const float rs = 1.f / sqrtf(wave_sum(ss) / (float)d + eps);
 #pragma unroll
       for (int u = 0; u < 4; ++u) y[u] *= rs;
@@ -606,9 +622,17 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
     else dst = slot_t >= 0 ? k_cache + (((int64_t)(slot_t / P) * Hkv + head) * P + slot_t % P) * D : nullptr;
     if (dst != nullptr) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int c = lane + 64 * u;
-        if (c < D) dst[c] = c < d ? (T)y[u] : (T)0.f;
+      for (int u = 0; u < 4; u += 2) {
+        const int c = (u >> 1) * 128 + 2 * lane;      // D is even, so a pair is inside or outside together
+        if (c < D) {
+          const T lo_v = c < d ? (T)y[u] : (T)0.f, hi_v = c + 1 < d ? (T)y[u + 1] : (T)0.f;
+          if constexpr (sizeof(T) == 2) {
+            *reinterpret_cast<bf16x2*>(dst + c) = bf16x2{(bf16)lo_v, (bf16)hi_v};
+          } else {
+            dst[c] = lo_v;
+            dst[c + 1] = hi_v;
+          }
+        }
       }
     }
   }
@@ -629,14 +653,14 @@ OME_API int ome_conv_rope_cache(const void* q, int64_t q_stride, const void* k, 
   if (tiles > 65535) return -3;
   const int dmax = dim > vdim ? dim : vdim;
   const size_t lds = (size_t)((CR_TILE + (K > 0 ? K - 1 : 0)) * dmax + K * dmax) * sizeof(float);
-  if (lds > 160 * 1024) return -3;
+  if (lds > 150 * 1024) return -3;   // (the staged sequence starts take 4 KB of static LDS beside it)
   dim3 grid(Hq + 2 * Hkv, tiles);
 #define CRC_LAUNCH(TT)                                                                                              \
   do {                                                                                                              \
     static bool big_ = false; /* once: allow the largest dynamic LDS block */                                       \
     if (lds > 64 * 1024 && !big_) {                                                                                \
       hipError_t e_ = hipFuncSetAttribute((const void*)conv_rope_cache_kernel<TT>,                                                \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);                \
       if (e_ != hipSuccess) return (int)e_;                                                                        \
       big_ = true;                                                                                                 \
     }                                                                                                              \

@@ -276,7 +276,13 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
     const int* __restrict__ kv_lens, const int2* __restrict__ items, const bf16* __restrict__ gate,
     int64_t gate_stride, bf16* __restrict__ out, int64_t out_stride, int H, int Hkv, int vdim, float mul, int window,
     const float* __restrict__ sinks, const float* __restrict__ r1, const float* __restrict__ r2,
-    const float* __restrict__ talk) {
+    const float* __restrict__ talk, int mode, int chunk, int RT, float* __restrict__ part_ml,
+    float* __restrict__ part_o) {
+  // mode 0: both passes over all keys.  Split keys (single rows with long contexts: few rows, so
+  // the keys of a row are spread over gridDim.z workgroups of `chunk` keys each): mode 1 = pass 1 of
+  // this workgroup's keys, raw (m, l) to part_ml; mode 2 = (m, l) merged over the splits (+ sink),
+  // pass 2 of this workgroup's keys, fp32 partial outputs to part_o (they simply add up: the
+  // weights are final).  Partials are indexed [tile][split][head][row < RT].
   constexpr int P = 16, NB = D / 16, KS = D / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int HP = (H + 31) & ~31;          // heads as a k dimension
@@ -298,9 +304,11 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int n = lane & 15, g = lane >> 4;
   const int r_hi = min(r0 + 16, q_len);
-  const int kv_end = min(kv_len, prefix + r_hi);
   const int lo0 = window > 0 ? max(0, prefix + r0 - window + 1) : 0;
-  const int kv_lo = lo0 & ~31;
+  const int Z = gridDim.z, z = blockIdx.z;
+  const int kv_lo = (lo0 & ~31) + (mode ? z * chunk : 0);
+  const int kv_end = mode ? min(min(kv_len, prefix + r_hi), kv_lo + chunk) : min(kv_len, prefix + r_hi);
+  const int64_t tile = (int64_t)blockIdx.x * gridDim.y + blockIdx.y;
   const int* bt = block_tables + (int64_t)s * bt_stride;
   const int64_t kpage = (int64_t)Hkv * P * D;
   const int r = r0 + n;                       // this lane's query row
@@ -308,14 +316,30 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
   const int qpos = prefix + r;
   const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
 
-  for (int i = threadIdx.x; i < HM * ldb; i += blockDim.x) {   // talk as bf16, zero padded
-    const int h = i / ldb, c = i - h * ldb;
-    Tk[i] = (bf16)((h < H && c < H) ? talk[h * H + c] : 0.f);
+  if (mode != 1) {
+    for (int i = threadIdx.x; i < HM * ldb; i += blockDim.x) {   // talk as bf16, zero padded
+      const int h = i / ldb, c = i - h * ldb;
+      Tk[i] = (bf16)((h < H && c < H) ? talk[h * H + c] : 0.f);
+    }
+    for (int i = threadIdx.x; i < 512 * ldb; i += blockDim.x) Pb[i] = (bf16)0.f;   // (pad heads stay zero)
   }
-  for (int i = threadIdx.x; i < 512 * ldb; i += blockDim.x) Pb[i] = (bf16)0.f;   // (pad heads stay zero)
+  if (mode == 2) {   // (m, l) of every head and row over all splits
+    for (int i = threadIdx.x; i < H * RT; i += blockDim.x) {
+      const int head = i / RT, nn = i - head * RT;
+      float m = sinks != nullptr ? sinks[head] * 1.4426950408889634f : -__builtin_inff();
+      for (int zz = 0; zz < Z; ++zz) m = fmaxf(m, part_ml[(((tile * Z + zz) * H + head) * RT + nn) * 2]);
+      float l = sinks != nullptr ? __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - m) : 0.f;
+      for (int zz = 0; zz < Z; ++zz) {
+        const float* pz = part_ml + (((tile * Z + zz) * H + head) * RT + nn) * 2;
+        if (pz[1] > 0.f) l += pz[1] * __builtin_amdgcn_exp2f(pz[0] - m);
+      }
+      ml[(head * 16 + nn) * 2] = (m == -__builtin_inff()) ? 0.f : m;
+      ml[(head * 16 + nn) * 2 + 1] = l > 0.f ? 1.f / l : 0.f;
+    }
+  }
 
   // ---- pass 1
-  for (int j = 0; j < HPW; ++j) {
+  for (int j = 0; j < HPW && mode != 2; ++j) {
     const int head = wave + NW * j;
     if (head >= H) break;
     const int kvh = head / G;
@@ -359,6 +383,14 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
       l_i = l_i * __builtin_amdgcn_exp2f(m_i - m_use) + rs;
       m_i = m_new;
     }
+    if (mode == 1) {
+      if (g == 0 && n < RT) {
+        float* pz = part_ml + (((tile * Z + z) * H + head) * RT + n) * 2;
+        pz[0] = m_i;
+        pz[1] = l_i;
+      }
+      continue;
+    }
     if (sinks != nullptr) {
       const float sk = sinks[head] * 1.4426950408889634f;
       const float m_new = fmaxf(m_i, sk);
@@ -370,6 +402,7 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
       ml[(head * 16 + n) * 2 + 1] = l_i > 0.f ? 1.f / l_i : 0.f;
     }
   }
+  if (mode == 1) return;
   __syncthreads();
 
   // ---- pass 2
@@ -442,6 +475,21 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
     // (the next tile's (a) writes Pb only, and its (b) follows a barrier after this tile's (c))
   }
   // ---- epilogue: O^T lane (row n, dims 16 nb + 4 g + i), times the head's gate
+  if (mode == 2) {
+    if (row_ok && n < RT) {
+#pragma unroll
+      for (int j = 0; j < HPW; ++j) {
+        const int head = wave + NW * j;
+        if (head < H) {
+          float* po = part_o + (((tile * Z + z) * H + head) * RT + n) * D;
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+            *reinterpret_cast<f32x4*>(po + 16 * nb + 4 * g) = o[j][nb];
+        }
+      }
+    }
+    return;
+  }
   if (row_ok) {
 #pragma unroll
     for (int j = 0; j < HPW; ++j) {
@@ -462,6 +510,21 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
   }
 }
 
+// out[b, h * vdim + d] = gate(b, h) * sum over splits of part_o[b][z][h][d]   (single rows: RT = 1)
+__global__ __launch_bounds__(256) void talking_combine_kernel(const float* __restrict__ part_o, int Z, int H, int D,
+                                                              int vdim, const bf16* __restrict__ gate,
+                                                              int64_t gate_stride, bf16* __restrict__ out,
+                                                              int64_t out_stride) {
+  const int64_t b = blockIdx.x;
+  for (int o = threadIdx.x; o < H * vdim; o += 256) {
+    const int h = o / vdim, d = o - h * vdim;
+    float a = 0.f;
+    for (int z = 0; z < Z; ++z) a += part_o[(((b * Z + z) * H + h)) * D + d];
+    if (gate != nullptr) a *= 1.f / (1.f + __expf(-(float)gate[b * gate_stride + h]));
+    out[b * out_stride + o] = (bf16)a;
+  }
+}
+
 }  // namespace
 
 // items int32 [n_items, 2] = (sequence, first row) of `item_rows`-row work items (a multiple of 16);
@@ -471,8 +534,12 @@ OME_API int ome_talking_prefill(const void* q, int64_t q_stride, const void* k_c
                                 const int* items, int n_items, int item_rows, const void* gate, int64_t gate_stride,
                                 void* out, int64_t out_stride, int H, int Hkv, int D, int vdim, int P, float scale,
                                 int window, const float* sinks, const float* r1, const float* r2, const float* talk,
-                                hipStream_t stream) {
+                                int splits, int chunk, float* part_ml, float* part_o, hipStream_t stream) {
+  // splits > 1 (item_rows must be 16, every sequence brings ONE row: decode): keys in `splits`
+  // pieces of `chunk` (a multiple of 32) per row; part_ml fp32 [n_items, splits, H, 2], part_o fp32
+  // [n_items, splits, H, D]
   if (n_items <= 0) return 0;
+  if (splits > 1 && (item_rows != 16 || chunk <= 0 || chunk % 32 || part_ml == nullptr || part_o == nullptr)) return -2;
   if (P != 16 || H <= 0 || Hkv <= 0 || H % Hkv || vdim <= 0 || vdim > D || item_rows <= 0 || item_rows % 16 ||
       (q_stride & 7) || r1 == nullptr || r2 == nullptr || talk == nullptr)
     return -2;
@@ -482,7 +549,7 @@ OME_API int ome_talking_prefill(const void* q, int64_t q_stride, const void* k_c
   const int HP = (H + 31) & ~31, HM = (H + 15) & ~15, ldb = HP + TP_PAD, ldm = 32 + TP_PAD;
   const size_t lds = (size_t)(512 * ldb + H * 16 * ldm + HM * ldb) * 2 + (size_t)H * 16 * 2 * 4;
   if (lds > 160 * 1024) return -3;
-  const dim3 grid(n_items, item_rows / 16);
+  const dim3 grid(n_items, item_rows / 16), gridz(n_items, 1, splits > 1 ? splits : 1);
   const float mul = scale * 1.4426950408889634f;
 #define TP_LAUNCH(DD, HH)                                                                                            \
   do {                                                                                                               \
@@ -493,10 +560,20 @@ OME_API int ome_talking_prefill(const void* q, int64_t q_stride, const void* k_c
       if (e_ != hipSuccess) return (int)e_;                                                                          \
       big_ = true;                                                                                                   \
     }                                                                                                                \
-    talking_prefill_kernel<DD, HH><<<grid, 64 * NW, lds, stream>>>(                                                  \
-        (const bf16*)q, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, bt_stride, cu_q, kv_lens, \
-        (const int2*)items, (const bf16*)gate, gate_stride, (bf16*)out, out_stride, H, Hkv, vdim, mul, window, sinks, \
-        r1, r2, talk);                                                                                               \
+    if (splits > 1) {                                                                                                \
+      for (int md = 1; md <= 2; ++md)                                                                                \
+        talking_prefill_kernel<DD, HH><<<gridz, 64 * NW, md == 1 ? 0 : lds, stream>>>(                               \
+            (const bf16*)q, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, bt_stride, cu_q,     \
+            kv_lens, (const int2*)items, (const bf16*)gate, gate_stride, (bf16*)out, out_stride, H, Hkv, vdim, mul,  \
+            window, sinks, r1, r2, talk, md, chunk, 1, part_ml, part_o);                                             \
+      talking_combine_kernel<<<n_items, 256, 0, stream>>>(part_o, splits, H, DD, vdim, (const bf16*)gate,            \
+                                                          gate_stride, (bf16*)out, out_stride);                      \
+    } else {                                                                                                         \
+      talking_prefill_kernel<DD, HH><<<grid, 64 * NW, lds, stream>>>(                                                \
+          (const bf16*)q, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, bt_stride, cu_q,       \
+          kv_lens, (const int2*)items, (const bf16*)gate, gate_stride, (bf16*)out, out_stride, H, Hkv, vdim, mul,    \
+          window, sinks, r1, r2, talk, 0, 0, 16, nullptr, nullptr);                                                  \
+    }                                                                                                                \
   } while (0)
   if (D == 64) TP_LAUNCH(64, 4);
   else if (D == 128) TP_LAUNCH(128, 4);

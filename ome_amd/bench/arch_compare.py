@@ -486,9 +486,13 @@ def kernel_table_milenex(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
     rows_i = torch.arange(B, dtype=torch.int32, device=dev)
     kvb = B * Hkv * D * 2 * 2 * W
     pair("talking_attn decode 64 x 4096 ctx, window 1024",
+         lambda: ops.talking_decode(q, kc, vc, bt, sl, 0.09, W, sinks, r1, r2, talk, gate, D),
+         lambda: ops.paged_decode(q, kc, vc, bt, sl, 0.09, ws, W, sinks=sinks), kvb, kvb,
+         "three launches: pass 1 per key split, pass 2 per key split (keys read again, mix over heads), sum + gate", 10)
+    pair("talking_attn row kernel (fp32 models' path, here on bf16), same shape",
          lambda: ops.talking_attn(q, kc, vc, bt, rows_i, sl - 1, 0.09, W, sinks, r1, r2, talk, gate, D),
          lambda: ops.paged_decode(q, kc, vc, bt, sl, 0.09, ws, W, sinks=sinks), kvb, kvb,
-         "all heads of a row in one workgroup (the mix needs every head's final weight)", 10)
+         "exactness path: one workgroup per row, no matrix cores", 3)
     # ---- prefill, 2 x 2048 rows
     q_lens = [2048, 2048]
     Tq = sum(q_lens)
@@ -498,10 +502,8 @@ def kernel_table_milenex(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
     kl = torch.tensor(q_lens, dtype=torch.int32, device=dev)
     bt2 = (torch.arange(2 * 128, dtype=torch.int32, device=dev) + 1).view(2, 128)
     items = torch.tensor(ops.prefill_work_items(q_lens, q_lens), dtype=torch.int32, device=dev)
-    tok_row = torch.arange(Tq, dtype=torch.int32, device=dev) // 2048
-    tok_pos = (torch.arange(Tq, dtype=torch.int32, device=dev) % 2048).to(torch.int32)
     flops = 4.0 * Hq * D * sum(min(W, i + 1) for i in range(2048)) * 2
-    tn = _time_us(lambda: ops.talking_attn(qp, kc, vc, bt2, tok_row, tok_pos, 0.09, W, sinks, r1, r2, talk, gp, D), 5)
+    tn = _time_us(lambda: ops.talking_prefill(qp, kc, vc, bt2, cu, kl, items, 0.09, W, sinks, r1, r2, talk, gp, D), 5)
     tl = _time_us(lambda: ops.paged_prefill(qp, kc, vc, bt2, cu, kl, items, 0.09, W, sinks=sinks), 5)
     rows.append({"kernel": "talking_attn prefill 2 x 2048 rows, window 1024", "us": round(tn, 1),
                  "roofline": round(flops / tn / 1e6 / 2.5e3, 3), "like_us": round(tl, 1),

@@ -643,18 +643,18 @@ class TalkingHeadsAttention(_Block):
         o = torch.empty(T, self.Hq * self.vdim, dtype=h.dtype, device=h.device)
         gate = p[:, nq + nk + nv:]
         meta = ctx.meta
-        n = 0 if meta.is_decode else (meta.num_prefill if meta.mode == "mixed" else T)
-        if n and ops.talking_prefill_ok(q, self.Hq, self.D, k_cache.shape[2]):   # prompt chunks: the MFMA kernel
-            ops.talking_prefill(q[:n], k_cache, v_cache, meta.block_tables, meta.cu_q, meta.kv_lens, meta.items,
-                                self.scale, self.window, self.sink, self.r1, self.r2, self.talk, gate[:n], self.vdim,
-                                out=o[:n])
-        else:
-            n = 0
-        if n < T:                              # single rows (and every row of fp32 models): the row kernel
+        args = (self.scale, self.window, self.sink, self.r1, self.r2, self.talk)
+        if ops.talking_prefill_ok(q, self.Hq, self.D, k_cache.shape[2]):   # bf16: the MFMA kernels
+            n = 0 if meta.is_decode else (meta.num_prefill if meta.mode == "mixed" else T)
+            if n:                              # prompt chunks: 16 rows x all heads per workgroup
+                ops.talking_prefill(q[:n], k_cache, v_cache, meta.block_tables, meta.cu_q, meta.kv_lens, meta.items,
+                                    *args, gate[:n], self.vdim, out=o[:n])
+            if n < T:                          # single rows: the keys of a row split over workgroups
+                bt = meta.block_tables if meta.is_decode else meta.dec_block_tables
+                ops.talking_decode(q[n:], k_cache, v_cache, bt, meta.seq_lens, *args, gate[n:], self.vdim, out=o[n:])
+        else:                                  # fp32 models, shapes without an MFMA kernel, the CPU: the row kernel
             for s, e, bt, rows, pos in attention_rows(meta, T):
-                if e > n:
-                    ops.talking_attn(q[s:e], k_cache, v_cache, bt, rows, pos, self.scale, self.window, self.sink,
-                                     self.r1, self.r2, self.talk, gate[s:e], self.vdim, out=o[s:e])
+                ops.talking_attn(q[s:e], k_cache, v_cache, bt, rows, pos, *args, gate[s:e], self.vdim, out=o[s:e])
         return linear(o, self.w_o)
 
 

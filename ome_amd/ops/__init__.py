@@ -2050,5 +2050,49 @@ def talking_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
          _i32(block_tables).data_ptr(), block_tables.stride(0), _i32(cu_q).data_ptr(), _i32(kv_lens).data_ptr(),
          _i32(items).data_ptr(), items.shape[0], int(rows), ptr(gate), gate.stride(0) if gate is not None else 0,
          out.data_ptr(), out.stride(0), H, Hkv, D, vdim, P, float(scale), int(window), _sinks(sinks), r1.data_ptr(),
-         r2.data_ptr(), talk.data_ptr(), stream_ptr())
+         r2.data_ptr(), talk.data_ptr(), 1, 0, None, None, stream_ptr())
+    return out
+
+
+_TD_IDX: dict = {}
+
+
+def talking_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                   seq_lens: torch.Tensor, scale: float, window: int, sinks: torch.Tensor | None, r1: torch.Tensor,
+                   r2: torch.Tensor, talk: torch.Tensor, gate: torch.Tensor | None, vdim: int,
+                   out: torch.Tensor | None = None) -> torch.Tensor:
+    """:func:`talking_attn` for single rows: row b is the last token of sequence b (``seq_lens``
+    includes it).  bf16 on the GPU with a shape of :func:`talking_prefill_ok`: the MFMA kernel with
+    a row's keys split over several workgroups (few rows must still fill the chip) -- pass 1 per
+    split, then pass 2 per split with the merged maxima and sums, then the sum of the partial
+    outputs times the gate; the split is a function of the shapes only, so the launches can be
+    captured.  Anything else: the row kernel."""
+    B, H, D = q.shape
+    Hkv, P = k_cache.shape[1], k_cache.shape[2]
+    out = torch.empty(B, H * vdim, dtype=q.dtype, device=q.device) if out is None else out
+    if not talking_prefill_ok(q, H, D, P):
+        return talking_attn(q, k_cache, v_cache, block_tables, torch.arange(B, dtype=torch.int32, device=q.device),
+                            _i32(seq_lens) - 1, scale, window, sinks, r1, r2, talk, gate, vdim, out)
+    key = (q.device, B)
+    idx = _TD_IDX.get(key)
+    if idx is None:      # cu_q = 0 .. B, items = (b, 0): kept (captured graphs read them again)
+        ar = torch.arange(B + 1, dtype=torch.int32, device=q.device)
+        idx = _TD_IDX[key] = (ar, torch.stack([ar[:B], torch.zeros_like(ar[:B])], 1).contiguous())
+    cu, items = idx
+    span = block_tables.shape[1] * P
+    if window > 0:
+        span = min(span, window + 32)
+    splits = max(1, min(-(-256 // B), span // 64, 32))
+    chunk = -(-(-(-span // splits)) // 32) * 32
+    assert q.stride(2) == 1 and q.stride(1) == D and k_cache.shape[3] == D and out.stride(1) == 1
+    assert gate is None or (gate.stride(1) == 1 and gate.dtype == q.dtype)
+    pml = po = None
+    if splits > 1:
+        pml = torch.empty(B * splits * H * 2, dtype=torch.float32, device=q.device)
+        po = torch.empty(B * splits * H * D, dtype=torch.float32, device=q.device)
+    call("ome_talking_prefill", q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(),
+         _i32(block_tables).data_ptr(), block_tables.stride(0), cu.data_ptr(), _i32(seq_lens).data_ptr(),
+         items.data_ptr(), B, 16, ptr(gate), gate.stride(0) if gate is not None else 0, out.data_ptr(), out.stride(0),
+         H, Hkv, D, vdim, P, float(scale), int(window), _sinks(sinks), r1.data_ptr(), r2.data_ptr(), talk.data_ptr(),
+         splits, chunk, ptr(pml), ptr(po), stream_ptr())
     return out

@@ -156,6 +156,35 @@ def test_talking_prefill_kernel(H, Hkv, D, vdim, window):
     _close(got, want, BF, want.float().abs().max().item())
 
 
+@pytest.mark.parametrize("H,Hkv,D,vdim,window,ctx,B", [(6, 3, 64, 64, 136, 400, 4), (32, 8, 128, 128, 1024, 2100, 3),
+                                                       (4, 1, 64, 7, 6, 33, 2), (16, 2, 256, 200, 0, 700, 5),
+                                                       (12, 4, 128, 96, 0, 90, 70), (1, 1, 64, 64, 40, 50, 300)])
+def test_talking_decode_kernel(H, Hkv, D, vdim, window, ctx, B):
+    """Single rows with their keys split over workgroups (contexts of unequal length, one of a
+    single token, a padding row of length 0) against the row reference."""
+    g = torch.Generator().manual_seed(H + ctx)
+    P = 16
+    n_pages = -(-ctx // P)
+    kc = (torch.randn(B * n_pages + 2, Hkv, P, D, generator=g) * 0.5).to(BF)
+    vc = torch.randn(B * n_pages + 2, Hkv, D, P, generator=g).to(BF)
+    bt = (torch.randperm(B * n_pages, generator=g) + 1).view(B, n_pages).to(torch.int32)
+    lens = torch.randint(1, ctx + 1, (B,), generator=g).to(torch.int32)
+    lens[0], lens[-1] = ctx, 1
+    if B > 2:
+        lens[1] = 0
+    q = (torch.randn(B, H, D, generator=g) * 0.5).to(BF)
+    gate = torch.randn(B, H + 5, generator=g).to(BF)
+    r1, r2 = torch.rand(H, generator=g), torch.rand(H, generator=g) * 2 + 0.1
+    talk = (torch.eye(H) + torch.randn(H, H, generator=g) * 0.3).to(BF).float()
+    sinks = torch.randn(H, generator=g)
+    seq = torch.arange(B, dtype=torch.int32)
+    want = ops.talking_attn(q, kc, vc, bt, seq, lens - 1, 0.2, window, sinks, r1, r2, talk, gate[:, :H], vdim)
+    d = lambda t: t.to(DEV)   # noqa: E731
+    got = ops.talking_decode(d(q), d(kc), d(vc), d(bt), d(lens), 0.2, window, d(sinks), d(r1), d(r2), d(talk),
+                             d(gate)[:, :H], vdim)
+    _close(got, want, BF, want.float().abs().max().item())
+
+
 @pytest.mark.parametrize("dt", DTYPES)
 def test_small_ops(dt):
     g = torch.Generator().manual_seed(2)
