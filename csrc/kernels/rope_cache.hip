@@ -488,7 +488,7 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
     z -= n;
   }
   if (s >= S) return;
-  const int r0 = cu[s], r1 = cu[s + 1];
+  const int r0 = cus[s], r1 = cus[s + 1];
   const int a = r0 + z * CR_TILE;
   const int e = min(a + CR_TILE, r1);
   const int kind = hh < Hq ? 0 : (hh < Hq + Hkv ? 1 : 2);
@@ -503,31 +503,75 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
   float* rows = sm;
   float* taps = sm + (CR_TILE + KT) * d;
   const int tid = threadIdx.x;
-  for (int i = tid; i < K * d; i += 256) taps[i] = (float)wt[(int64_t)(head * d + i % d) * K + i / d];   // [j][c]
+  const int wave = tid >> 6, lane = tid & 63;
+  // A global load costs a round trip of a microsecond under load, so the kernel is arranged as a few
+  // rounds of independent loads: (1) the rows' positions / cache slots (lane i of a wave holds row
+  // wave + 4 i of the tile) together with the sequence's slot and the input rows and taps, (2) the
+  // rows' cos / sin, all asked for before the row loop, which then runs out of LDS and registers.
+  constexpr int RPW = CR_TILE / 4;   // rows per wave
+  int my_pos = 0, my_slot = -1;
+  if (lane < RPW && a + wave + 4 * lane < e) {
+    my_pos = positions[a + wave + 4 * lane];
+    my_slot = slots[a + wave + 4 * lane];
+  }
   T* tl = KT > 0 ? tail + (int64_t)slot[s] * KT * C + c0 : nullptr;
   const bool fresh = reset[s] != 0;
+  for (int i = tid; i < K * d; i += 256) taps[i] = (float)wt[(int64_t)(head * d + i % d) * K + i / d];   // [j][c]
   // input rows a - KT .. e - 1 of the sequence (before r0: the old tail, or zeros)
   const bool vec = sizeof(T) == 2 && (d & 7) == 0 && (sstride & 7) == 0 && (C & 7) == 0 &&
                    ((uintptr_t)src & 15) == 0 && (tl == nullptr || ((uintptr_t)tl & 15) == 0);
   if (vec) {
     const int cpr = d >> 3;   // 16-byte pieces per row
-    for (int i = tid; i < (e - a + KT) * cpr; i += 256) {
-      const int rr = i / cpr, c = (i - rr * cpr) << 3;
-      const int r = a - KT + rr;
-      bf16x8 x = {};
-      if (r >= r0) x = ld8((const bf16*)src + (int64_t)r * sstride + head * d + c);
-      else if (!fresh) x = ld8((const bf16*)tl + (int64_t)(KT + (r - r0)) * C + c);
+    const int total = (e - a + KT) * cpr;
+    for (int base = 0; base < total; base += 256 * 4) {
+      bf16x8 x[4];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) rows[rr * d + c + j] = (float)x[j];
+      for (int u = 0; u < 4; ++u) {   // all loads of the round first
+        const int i = base + tid + 256 * u;
+        x[u] = bf16x8{};
+        if (i < total) {
+          const int rr = i / cpr, c = (i - rr * cpr) << 3;
+          const int r = a - KT + rr;
+          if (r >= r0) x[u] = ld8((const bf16*)src + (int64_t)r * sstride + head * d + c);
+          else if (!fresh) x[u] = ld8((const bf16*)tl + (int64_t)(KT + (r - r0)) * C + c);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = base + tid + 256 * u;
+        if (i < total) {
+          const int rr = i / cpr, c = (i - rr * cpr) << 3;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) rows[rr * d + c + j] = (float)x[u][j];
+        }
+      }
     }
-  } else
-  for (int i = tid; i < (e - a + KT) * d; i += 256) {
-    const int rr = i / d, c = i - rr * d;
-    const int r = a - KT + rr;
-    float x;
-    if (r >= r0) x = (float)src[(int64_t)r * sstride + head * d + c];
-    else x = fresh ? 0.f : (float)tl[(int64_t)(KT + (r - r0)) * C + c];
-    rows[rr * d + c] = x;
+  } else {
+    for (int i = tid; i < (e - a + KT) * d; i += 256) {
+      const int rr = i / d, c = i - rr * d;
+      const int r = a - KT + rr;
+      float x;
+      if (r >= r0) x = (float)src[(int64_t)r * sstride + head * d + c];
+      else x = fresh ? 0.f : (float)tl[(int64_t)(KT + (r - r0)) * C + c];
+      rows[rr * d + c] = x;
+    }
+  }
+  // cos / sin of this wave's rows: lane -> pairs 2 lane (, 128 + 2 lane) -> table columns lane (, 64 + lane)
+  const int half = rot_dim >> 1;
+  float co[RPW][2], si[RPW][2];
+  if (kind != 2 && rot_dim > 0 && interleaved) {
+#pragma unroll
+    for (int it = 0; it < RPW; ++it) {
+      const int pos = __shfl(my_pos, it);
+      const float* cs = cos_sin + (int64_t)pos * rot_dim;
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const int ci = 64 * pr + lane;   // pair index
+        const bool on = 2 * ci < rot_dim && a + wave + 4 * it < e;
+        co[it][pr] = on ? cs[ci] : 1.f;
+        si[it][pr] = on ? cs[half + ci] : 0.f;
+      }
+    }
   }
   __syncthreads();
   if (z == 0 && KT > 0) {   // new tail: inputs L - KT .. L - 1 of the step; negative = old tail rows
@@ -538,12 +582,15 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
       tl[(int64_t)j * C + c] = t >= 0 ? src[(int64_t)(r0 + t) * sstride + head * d + c] : (T)rows[(KT + t) * d + c];
     }
   }
-  const int wave = tid >> 6, lane = tid & 63;
-  const int half = rot_dim >> 1;
   // a lane owns two pairs of neighbouring channels: register u <-> channel (u >> 1) * 128 + 2 lane + (u & 1)
   // (d <= 256), so an interleaved rotary pair sits in one lane and stores are 4 bytes wide
-  for (int r = a + wave; r < e; r += 4) {
-    const int rr = r - a;   // output row rr reads input rows rr .. rr + KT
+#pragma unroll
+  for (int it = 0; it < RPW; ++it) {
+    const int rr = wave + 4 * it;   // output row rr reads input rows rr .. rr + KT
+    const int r = a + rr;
+    const int slot_t = __shfl(my_slot, it);
+    const int pos = __shfl(my_pos, it);
+    if (r >= e) continue;
     float y[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -557,7 +604,6 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
       }
       y[u] = acc;
     }
-    const int slot_t = slots[r];
     if (kind == 2) {
       if (slot_t >= 0) {
         T* vc = v_cache + (((int64_t)(slot_t / P) * Hkv + head) * D) * P + slot_t % P;
@@ -570,20 +616,16 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
       continue;
     }
     if (rot_dim > 0) {
-      const float* cs = cos_sin + (int64_t)positions[r] * rot_dim;
       if (interleaved) {
 #pragma unroll
         for (int u = 0; u < 4; u += 2) {
-          const int c = (u >> 1) * 128 + 2 * lane;
-          if (c < rot_dim) {
-            const float co = cs[c >> 1], si = cs[half + (c >> 1)];
-            const float ev = y[u], od = y[u + 1];
-            y[u] = ev * co - od * si;
-            y[u + 1] = od * co + ev * si;
-          }
+          const float ev = y[u], od = y[u + 1];
+          y[u] = ev * co[it][u >> 1] - od * si[it][u >> 1];
+          y[u + 1] = od * co[it][u >> 1] + ev * si[it][u >> 1];
         }
       } else {   // channel i pairs with i + half: the partner pc sits in lane (pc & 127) >> 1, register
         // (pc >> 7) * 2 + (pc & 1)
+        const float* cs = cos_sin + (int64_t)pos * rot_dim;
         float other[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -603,8 +645,8 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
           const int c = (u >> 1) * 128 + 2 * lane + (u & 1);
           if (c < rot_dim) {
             const int i = c < half ? c : c - half;
-            const float co = cs[i], si = cs[half + i];
-            y[u] = c < half ? y[u] * co - other[u] * si : y[u] * co + other[u] * si;
+            const float cc = cs[i], ss = cs[half + i];
+            y[u] = c < half ? y[u] * cc - other[u] * ss : y[u] * cc + other[u] * ss;
           }
         }
       }

@@ -239,8 +239,8 @@ OME_API int ome_talking_attn(const void* q, int64_t q_stride, const void* k_cach
 
 // ------------------------------------------------------------------------------------------
 // Prompt chunks on the matrix cores (bf16).  One workgroup = 16 consecutive query rows of one
-// sequence (a quarter / half of a prefill work item) x ALL heads; wave w owns heads w, w + NW, ...
-// (at most HPW of them, NW = waves of the workgroup).  Keys go by in tiles of 32 (two pages):
+// sequence (a quarter / half of a prefill work item) x ALL heads; wave w owns the HPW consecutive
+// heads from w * HPW (heads of one kv head share its key and value fragments).  Keys go by in tiles of 32 (two pages):
 //
 //   pass 1   per head: S^T = K Q^T (MFMA 16x16x32; lane (n, g) holds row n, keys 16X + 4g + i),
 //            bias, mask, running maximum and sum per row -> with the sink, m and 1 / l to LDS.
@@ -267,7 +267,12 @@ __device__ __forceinline__ bf16x8 ta_cat44(bf16x4 a, bf16x4 b) {
   return bf16x8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
 }
 
-constexpr int TP_PAD = 8;   // bf16 elements of padding per LDS row
+__device__ __forceinline__ bf16x8 ta_lds8(const bf16* p) {   // 8 elements from an 8-byte aligned LDS address
+  return ta_cat44(*reinterpret_cast<const bf16x4*>(p), *reinterpret_cast<const bf16x4*>(p + 4));
+}
+
+constexpr int TP_PAD = 4;   // bf16 elements of padding per LDS row: rows 72 B apart, so the 2-byte stores of 16 rows
+                            // hit 16 banks; fragments are read as two 8-byte halves
 
 template <int D, int HPW>
 __global__ __launch_bounds__(512) void talking_prefill_kernel(
@@ -316,6 +321,19 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
   const int qpos = prefix + r;
   const int lo = window > 0 ? max(0, qpos - window + 1) : 0;
 
+  const int kv0 = min(wave * HPW, H - 1) / G;
+  const bool uni = wave * HPW < H && kv0 == min(wave * HPW + HPW - 1, H - 1) / G;   // one kv head for this wave
+  auto load_k = [&](int kb, int kvh, bf16x8(&fa)[KS], bf16x8(&fb)[KS]) {   // lane (key n, dims 32 ks + 8 g ..)
+    const int pA = bt[kb / P];
+    const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
+    const bf16* kA = k_cache + pA * kpage + (int64_t)kvh * P * D;
+    const bf16* kB = k_cache + pB * kpage + (int64_t)kvh * P * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      fa[ks] = ld8(kA + n * D + 32 * ks + 8 * g);
+      fb[ks] = ld8(kB + n * D + 32 * ks + 8 * g);
+    }
+  };
   if (mode != 1) {
     for (int i = threadIdx.x; i < HM * ldb; i += blockDim.x) {   // talk as bf16, zero padded
       const int h = i / ldb, c = i - h * ldb;
@@ -338,68 +356,103 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
     }
   }
 
-  // ---- pass 1
-  for (int j = 0; j < HPW && mode != 2; ++j) {
-    const int head = wave + NW * j;
-    if (head >= H) break;
-    const int kvh = head / G;
-    bf16x8 qf[KS];
-    const bf16* qr = q + (int64_t)(q0 + min(r, q_len - 1)) * q_stride + (int64_t)head * D;
+  // ---- pass 1: key tiles outside, this wave's heads inside, so that heads of one kv head share the
+  // key fragments (a wave owns HPW consecutive heads)
+  if (mode != 2) {
+    bf16x8 qf[HPW][KS];
+    float m_i[HPW], l_i[HPW], b1[HPW], b2[HPW];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = ld8(qr + 32 * ks + 8 * g);
-    const float b1 = r1[head], b2 = r2[head];
-    float m_i = -__builtin_inff(), l_i = 0.f;
+    for (int j = 0; j < HPW; ++j) {
+      const int head = min(wave * HPW + j, H - 1);
+      const bf16* qr = q + (int64_t)(q0 + min(r, q_len - 1)) * q_stride + (int64_t)head * D;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qf[j][ks] = ld8(qr + 32 * ks + 8 * g);
+      m_i[j] = -__builtin_inff();
+      l_i[j] = 0.f;
+      b1[j] = r1[head];
+      b2[j] = r2[head];
+    }
+    // the key fragments of the next tile are loaded while this one is worked on (when all heads of
+    // the wave share one kv head; otherwise they are loaded in place, per kv head)
+    bf16x8 na[KS], nb8[KS];
+    if (uni && kv_lo < kv_end) load_k(kv_lo, kv0, na, nb8);
     for (int kb = kv_lo; kb < kv_end; kb += 32) {
-      const int pA = bt[kb / P];
-      const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
-      const bf16* kA = k_cache + pA * kpage + (int64_t)kvh * P * D;
-      const bf16* kB = k_cache + pB * kpage + (int64_t)kvh * P * D;
-      f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+      bf16x8 ka[KS], kb8[KS];
+      int kv_prev = -1;
+      if (uni) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        sc[0] = ta_mfma(ld8(kA + n * D + 32 * ks + 8 * g), qf[ks], sc[0]);
-        sc[1] = ta_mfma(ld8(kB + n * D + 32 * ks + 8 * g), qf[ks], sc[1]);
-      }
-      float mt = -__builtin_inff();
-#pragma unroll
-      for (int X = 0; X < 2; ++X)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = kb + 16 * X + 4 * g + i;
-          const bool ok = row_ok && key <= qpos && key >= lo;
-          const float v = ok ? sc[X][i] * mul - b1 * __log2f(1.f + b2 * (float)(qpos - key)) : -__builtin_inff();
-          sc[X][i] = v;
-          mt = fmaxf(mt, v);
+        for (int ks = 0; ks < KS; ++ks) {
+          ka[ks] = na[ks];
+          kb8[ks] = nb8[ks];
         }
-      mt = group4_max(mt);
-      const float m_new = fmaxf(m_i, mt);
-      const float m_use = (m_new == -__builtin_inff()) ? 0.f : m_new;
-      float rs = 0.f;
-#pragma unroll
-      for (int X = 0; X < 2; ++X)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rs += __builtin_amdgcn_exp2f(sc[X][i] - m_use);
-      rs = group4_sum(rs);
-      l_i = l_i * __builtin_amdgcn_exp2f(m_i - m_use) + rs;
-      m_i = m_new;
-    }
-    if (mode == 1) {
-      if (g == 0 && n < RT) {
-        float* pz = part_ml + (((tile * Z + z) * H + head) * RT + n) * 2;
-        pz[0] = m_i;
-        pz[1] = l_i;
+        if (kb + 32 < kv_end) load_k(kb + 32, kv0, na, nb8);
+        kv_prev = kv0;
       }
-      continue;
+#pragma unroll
+      for (int j = 0; j < HPW; ++j) {
+        const int head = wave * HPW + j;
+        if (head < H) {
+          const int kvh = head / G;
+          if (kvh != kv_prev) {
+            load_k(kb, kvh, ka, kb8);
+            kv_prev = kvh;
+          }
+          f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            sc[0] = ta_mfma(ka[ks], qf[j][ks], sc[0]);
+            sc[1] = ta_mfma(kb8[ks], qf[j][ks], sc[1]);
+          }
+          float mt = -__builtin_inff();
+#pragma unroll
+          for (int X = 0; X < 2; ++X)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = kb + 16 * X + 4 * g + i;
+              const bool ok = row_ok && key <= qpos && key >= lo;
+              const float v =
+                  ok ? sc[X][i] * mul - b1[j] * __log2f(1.f + b2[j] * (float)(qpos - key)) : -__builtin_inff();
+              sc[X][i] = v;
+              mt = fmaxf(mt, v);
+            }
+          mt = group4_max(mt);
+          const float m_new = fmaxf(m_i[j], mt);
+          const float m_use = (m_new == -__builtin_inff()) ? 0.f : m_new;
+          float rs = 0.f;
+#pragma unroll
+          for (int X = 0; X < 2; ++X)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) rs += __builtin_amdgcn_exp2f(sc[X][i] - m_use);
+          rs = group4_sum(rs);
+          l_i[j] = l_i[j] * __builtin_amdgcn_exp2f(m_i[j] - m_use) + rs;
+          m_i[j] = m_new;
+        }
+      }
     }
-    if (sinks != nullptr) {
-      const float sk = sinks[head] * 1.4426950408889634f;
-      const float m_new = fmaxf(m_i, sk);
-      l_i = l_i * __builtin_amdgcn_exp2f(m_i - m_new) + __builtin_amdgcn_exp2f(sk - m_new);
-      m_i = m_new;
-    }
-    if (g == 0) {
-      ml[(head * 16 + n) * 2] = (m_i == -__builtin_inff()) ? 0.f : m_i;
-      ml[(head * 16 + n) * 2 + 1] = l_i > 0.f ? 1.f / l_i : 0.f;
+#pragma unroll
+    for (int j = 0; j < HPW; ++j) {
+      const int head = wave * HPW + j;
+      if (head < H) {
+        if (mode == 1) {
+          if (g == 0 && n < RT) {
+            float* pz = part_ml + (((tile * Z + z) * H + head) * RT + n) * 2;
+            pz[0] = m_i[j];
+            pz[1] = l_i[j];
+          }
+        } else {
+          float mm = m_i[j], ll = l_i[j];
+          if (sinks != nullptr) {
+            const float sk = sinks[head] * 1.4426950408889634f;
+            const float m_new = fmaxf(mm, sk);
+            ll = ll * __builtin_amdgcn_exp2f(mm - m_new) + __builtin_amdgcn_exp2f(sk - m_new);
+            mm = m_new;
+          }
+          if (g == 0) {
+            ml[(head * 16 + n) * 2] = (mm == -__builtin_inff()) ? 0.f : mm;
+            ml[(head * 16 + n) * 2 + 1] = ll > 0.f ? 1.f / ll : 0.f;
+          }
+        }
+      }
     }
   }
   if (mode == 1) return;
@@ -414,33 +467,50 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
   for (int kb = kv_lo; kb < kv_end; kb += 32) {
     const int pA = bt[kb / P];
     const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
+    // the value fragments of this tile are asked for now and used in (c), two barriers later
+    bf16x8 vpre[NB];
+    if (uni) {
+      const bf16* vA = v_cache + pA * kpage + (int64_t)kv0 * D * P;
+      const bf16* vB = v_cache + pB * kpage + (int64_t)kv0 * D * P;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        vpre[nb] = ta_cat44(ld4(vA + (16 * nb + n) * P + 4 * g), ld4(vB + (16 * nb + n) * P + 4 * g));
+    }
     // (a) final weights of this wave's heads
-    for (int j = 0; j < HPW; ++j) {
-      const int head = wave + NW * j;
-      if (head >= H) break;
-      const int kvh = head / G;
-      const bf16* qr = q + (int64_t)(q0 + min(r, q_len - 1)) * q_stride + (int64_t)head * D;
-      const bf16* kA = k_cache + pA * kpage + (int64_t)kvh * P * D;
-      const bf16* kB = k_cache + pB * kpage + (int64_t)kvh * P * D;
-      f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+    {
+      bf16x8 ka[KS], kb8[KS];
+      int kv_prev = -1;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const bf16x8 qv = ld8(qr + 32 * ks + 8 * g);
-        sc[0] = ta_mfma(ld8(kA + n * D + 32 * ks + 8 * g), qv, sc[0]);
-        sc[1] = ta_mfma(ld8(kB + n * D + 32 * ks + 8 * g), qv, sc[1]);
-      }
-      const float b1 = r1[head], b2 = r2[head];
-      const float m = ml[(head * 16 + n) * 2], il = ml[(head * 16 + n) * 2 + 1];
+      for (int j = 0; j < HPW; ++j) {
+        const int head = wave * HPW + j;
+        if (head < H) {
+          const int kvh = head / G;
+          if (kvh != kv_prev) {
+            load_k(kb, kvh, ka, kb8);
+            kv_prev = kvh;
+          }
+          const bf16* qr = q + (int64_t)(q0 + min(r, q_len - 1)) * q_stride + (int64_t)head * D;
+          f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-      for (int X = 0; X < 2; ++X)
+          for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8 qv = ld8(qr + 32 * ks + 8 * g);
+            sc[0] = ta_mfma(ka[ks], qv, sc[0]);
+            sc[1] = ta_mfma(kb8[ks], qv, sc[1]);
+          }
+          const float b1 = r1[head], b2 = r2[head];
+          const float m = ml[(head * 16 + n) * 2], il = ml[(head * 16 + n) * 2 + 1];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = kb + 16 * X + 4 * g + i;
-          const bool ok = row_ok && key <= qpos && key >= lo;
-          const float v = sc[X][i] * mul - b1 * __log2f(1.f + b2 * (float)(qpos - key));
-          const float p = ok ? __builtin_amdgcn_exp2f(v - m) * il : 0.f;
-          Pb[((8 * g + 4 * X + i) * 16 + n) * ldb + head] = (bf16)p;
+          for (int X = 0; X < 2; ++X)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = kb + 16 * X + 4 * g + i;
+              const bool ok = row_ok && key <= qpos && key >= lo;
+              const float v = sc[X][i] * mul - b1 * __log2f(1.f + b2 * (float)(qpos - key));
+              const float p = ok ? __builtin_amdgcn_exp2f(v - m) * il : 0.f;
+              Pb[((8 * g + 4 * X + i) * 16 + n) * ldb + head] = (bf16)p;
+            }
         }
+      }
     }
     __syncthreads();
     // (b) mix over heads: one key slot (16 rows) per product column block
@@ -448,8 +518,8 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
       for (int mt = 0; mt < HM / 16; ++mt) {
         f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int ks = 0; ks < HP / 32; ++ks)
-          acc = ta_mfma(*reinterpret_cast<const bf16x8*>(Tk + (16 * mt + n) * ldb + 32 * ks + 8 * g),
-                        *reinterpret_cast<const bf16x8*>(Pb + (16 * t + n) * ldb + 32 * ks + 8 * g), acc);
+          acc = ta_mfma(ta_lds8(Tk + (16 * mt + n) * ldb + 32 * ks + 8 * g),
+                        ta_lds8(Pb + (16 * t + n) * ldb + 32 * ks + 8 * g), acc);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int h = 16 * mt + 4 * g + i;
@@ -458,18 +528,37 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
       }
     }
     __syncthreads();
-    // (c) values
-    for (int j = 0; j < HPW; ++j) {
-      const int head = wave + NW * j;
-      if (head >= H) break;
-      const int kvh = head / G;
-      const bf16* vA = v_cache + pA * kpage + (int64_t)kvh * D * P;
-      const bf16* vB = v_cache + pB * kpage + (int64_t)kvh * D * P;
-      const bf16x8 pb = *reinterpret_cast<const bf16x8*>(Pm + (head * 16 + n) * ldm + 8 * g);
+    // (c) values: a value fragment is loaded once per kv head and feeds all its heads of this wave
+    {
+      bf16x8 pb[HPW];
+#pragma unroll
+      for (int j = 0; j < HPW; ++j) {
+        const int head = min(wave * HPW + j, H - 1);
+        pb[j] = ta_lds8(Pm + (head * 16 + n) * ldm + 8 * g);
+      }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         const int dim = 16 * nb + n;
-        o[j][nb] = ta_mfma(ta_cat44(ld4(vA + dim * P + 4 * g), ld4(vB + dim * P + 4 * g)), pb, o[j][nb]);
+        bf16x8 va;
+        int kv_prev = -1;
+        if (uni) {
+          va = vpre[nb];
+          kv_prev = kv0;
+        }
+#pragma unroll
+        for (int j = 0; j < HPW; ++j) {
+          const int head = wave * HPW + j;
+          if (head < H) {
+            const int kvh = head / G;
+            if (kvh != kv_prev) {
+              const bf16* vA = v_cache + pA * kpage + (int64_t)kvh * D * P;
+              const bf16* vB = v_cache + pB * kpage + (int64_t)kvh * D * P;
+              va = ta_cat44(ld4(vA + dim * P + 4 * g), ld4(vB + dim * P + 4 * g));
+              kv_prev = kvh;
+            }
+            o[j][nb] = ta_mfma(va, pb[j], o[j][nb]);
+          }
+        }
       }
     }
     // (the next tile's (a) writes Pb only, and its (b) follows a barrier after this tile's (c))
@@ -479,7 +568,7 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
     if (row_ok && n < RT) {
 #pragma unroll
       for (int j = 0; j < HPW; ++j) {
-        const int head = wave + NW * j;
+        const int head = wave * HPW + j;
         if (head < H) {
           float* po = part_o + (((tile * Z + z) * H + head) * RT + n) * D;
 #pragma unroll
@@ -493,7 +582,7 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
   if (row_ok) {
 #pragma unroll
     for (int j = 0; j < HPW; ++j) {
-      const int head = wave + NW * j;
+      const int head = wave * HPW + j;
       if (head < H) {
         const float gt = gate != nullptr
                              ? 1.f / (1.f + __expf(-(float)gate[(int64_t)(q0 + r) * gate_stride + head])) : 1.f;
