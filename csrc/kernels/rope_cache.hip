@@ -681,6 +681,241 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
 }
 }  // namespace
 
+// ------------------------------------------------------------------------------------------
+// The same step for the common shapes (head widths in multiples of 8, up to CV_MAXK taps,
+// interleaved rotary pairs, 16-byte aligned rows), without LDS and without barriers: one item =
+// (row, head of q / k / v), a lane owns 8 neighbouring channels (D / 8 lanes per item), reads its K
+// input vectors straight from the projection rows (L1 / L2 keep the K-fold reuse) or, for rows
+// before the step's first, from the sequence's tail, and writes 16-byte vectors.  Per row the
+// caller gives the sequence's first row of the step (row_start) and its state slot (row_slot,
+// bit 30 set: the sequence starts here, its tail counts as zeros).  The tails are rewritten by
+// conv_tail_kernel AFTER this kernel (stream order), one thread per (sequence, channel), which
+// reads a channel's old tail before it writes the new one.
+// ------------------------------------------------------------------------------------------
+namespace {
+constexpr int CV_MAXK = 6;
+
+template <typename T>
+__device__ __forceinline__ void cv_ld8(const T* p, float (&f)[8]) {
+  if constexpr (sizeof(T) == 2) {
+    const bf16x8 t = ld8((const bf16*)p);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = (float)t[j];
+  } else {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+    f[0] = a[0]; f[1] = a[1]; f[2] = a[2]; f[3] = a[3];
+    f[4] = b[0]; f[5] = b[1]; f[6] = b[2]; f[7] = b[3];
+  }
+}
+template <typename T>
+__device__ __forceinline__ void cv_st8(T* p, const float (&f)[8]) {
+  if constexpr (sizeof(T) == 2) {
+    bf16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = (bf16)f[j];
+    st8((bf16*)p, o);
+  } else {
+    *reinterpret_cast<f32x4*>(p) = f32x4{f[0], f[1], f[2], f[3]};
+    *reinterpret_cast<f32x4*>(p + 4) = f32x4{f[4], f[5], f[6], f[7]};
+  }
+}
+
+// K = taps (0: no convolution); GS = lanes per item = D / 8
+template <typename T, int K, int GS>
+__global__ __launch_bounds__(256) void conv_rope_cache_vec_kernel(
+    const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride, const T* __restrict__ v,
+    int64_t v_stride, const T* __restrict__ wq, const T* __restrict__ wk, const T* __restrict__ wv,
+    const T* __restrict__ tail, const int* __restrict__ row_start, const int* __restrict__ row_slot,
+    const int* __restrict__ positions, const float* __restrict__ cos_sin, int rot_dim, int unit_norm, float eps,
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ slots, int Tn,
+    int Hq, int Hkv, int dim, int vdim, int P) {
+  constexpr int D = GS * 8, KT = K > 0 ? K - 1 : 0, KK = K > 0 ? K : 1;
+  const int Ht = Hq + 2 * Hkv;
+  const int64_t item = (int64_t)blockIdx.x * (256 / GS) + threadIdx.x / GS;
+  const int l = threadIdx.x % GS;
+  const bool live = item < (int64_t)Tn * Ht;
+  // items go row by row within a head: the items of a wave share the head's taps and overlap in the
+  // input rows they read (cache hits), and neighbouring lanes' rows are neighbours
+  const int hh = live ? (int)(item / Tn) : 0;
+  const int t = live ? (int)(item - (int64_t)hh * Tn) : 0;
+  const int kind = hh < Hq ? 0 : (hh < Hq + Hkv ? 1 : 2);
+  const int head = kind == 0 ? hh : (kind == 1 ? hh - Hq : hh - Hq - Hkv);
+  const int d = kind == 2 ? vdim : dim;
+  const T* src = kind == 0 ? q : (kind == 1 ? k : v);
+  const int64_t sstride = kind == 0 ? q_stride : (kind == 1 ? k_stride : v_stride);
+  const T* wt = kind == 0 ? wq : (kind == 1 ? wk : wv);
+  const int C = Hq * dim + Hkv * dim + Hkv * vdim;
+  const int c0 = kind == 0 ? head * dim : (kind == 1 ? Hq * dim + head * dim : (Hq + Hkv) * dim + head * vdim);
+  const int c8 = 8 * l;
+  const bool on = live && c8 < d;       // (d is a multiple of 8: a lane's channels are all inside or all outside)
+  // round 1: the row's sequence, position and cache slot
+  const int r0 = row_start[t], rs = row_slot[t], pos = positions[t], slot_t = slots[t];
+  const bool fresh = (rs >> 30) & 1;
+  const int st = rs & 0x3fffffff;
+  // round 2: inputs and taps
+  float x[KK][8], w[8 * KK];
+#pragma unroll
+  for (int j = 0; j < KK; ++j) {
+    const int r = t - KT + j;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[j][e] = 0.f;
+    if (on) {
+      if (r >= r0) cv_ld8<T>(src + (int64_t)r * sstride + head * d + c8, x[j]);
+      else if (!fresh) cv_ld8<T>(tail + ((int64_t)st * KT + (KT + r - r0)) * C + c0 + c8, x[j]);
+    }
+  }
+  float y[8];
+  if constexpr (K > 0) {
+    if (on) {   // this lane's taps are contiguous: w[e * K + j]
+#pragma unroll
+      for (int m = 0; m < K; ++m) {
+        float tmp[8];
+        cv_ld8<T>(wt + (int64_t)(head * d + c8) * K + 8 * m, tmp);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w[8 * m + e] = tmp[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < K; ++j) acc += w[e * K + j] * x[j][e];
+      y[e] = on ? acc : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = x[0][e];
+  }
+  if (kind == 2) {
+    if (on && slot_t >= 0) {
+      T* vc = v_cache + (((int64_t)(slot_t / P) * Hkv + head) * D + c8) * P + slot_t % P;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vc[(int64_t)e * P] = (T)y[e];
+    }
+  }
+  // (q / k from here; lanes of value items only take part in the shuffles)
+  if (kind != 2 && on && rot_dim > 0) {
+    const float* cs = cos_sin + (int64_t)pos * rot_dim;
+    const int half = rot_dim >> 1;
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      const int c = c8 + e;
+      if (c < rot_dim) {
+        const float co = cs[c >> 1], si = cs[half + (c >> 1)];
+        const float ev = y[e], od = y[e + 1];
+        y[e] = ev * co - od * si;
+        y[e + 1] = od * co + ev * si;
+      }
+    }
+  }
+  if (unit_norm) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += y[e] * y[e];
+#pragma unroll
+    for (int o = GS / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    const float rsq = 1.f / sqrtf(ss / (float)d + eps);
+    if (kind != 2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) y[e] *= rsq;
+    }
+  }
+  if (live && kind != 2) {   // every lane of the item writes its 16 bytes: zeros beyond the head's width
+    T* dst;
+    if (kind == 0) dst = q_out + ((int64_t)t * Hq + head) * D;
+    else dst = slot_t >= 0 ? k_cache + (((int64_t)(slot_t / P) * Hkv + head) * P + slot_t % P) * D : nullptr;
+    if (dst != nullptr) cv_st8<T>(dst + c8, y);
+  }
+}
+
+// new tail of every sequence: inputs L - KT .. L - 1 of the step (negative: the old tail, shifted)
+template <typename T>
+__global__ __launch_bounds__(256) void conv_tail_kernel(const T* __restrict__ q, int64_t q_stride,
+                                                        const T* __restrict__ k, int64_t k_stride,
+                                                        const T* __restrict__ v, int64_t v_stride,
+                                                        T* __restrict__ tail, const int* __restrict__ cu,
+                                                        const int* __restrict__ slot, const int* __restrict__ reset,
+                                                        int KT, int nq, int nk, int C) {
+  const int c = blockIdx.x * 256 + threadIdx.x, s = blockIdx.y;
+  if (c >= C) return;
+  const int r0 = cu[s], L = cu[s + 1] - r0;
+  if (L <= 0) return;
+  const T* src = c < nq ? q + c : (c < nq + nk ? k + (c - nq) : v + (c - nq - nk));
+  const int64_t stride = c < nq ? q_stride : (c < nq + nk ? k_stride : v_stride);
+  T* tl = tail + (int64_t)slot[s] * KT * C + c;
+  const bool fresh = reset[s] != 0;
+  T val[32];
+  for (int j = 0; j < KT; ++j) {
+    const int t = L - KT + j;
+    val[j] = t >= 0 ? src[(int64_t)(r0 + t) * stride] : (fresh ? (T)0.f : tl[(int64_t)(j + L) * C]);
+  }
+  for (int j = 0; j < KT; ++j) tl[(int64_t)j * C] = val[j];
+}
+}  // namespace
+
+// Fast path of ome_conv_rope_cache (see conv_rope_cache_vec_kernel).  Returns -9 when the shapes
+// are not the ones it is built for: the caller then takes the general kernel.
+OME_API int ome_conv_rope_cache_vec(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                                    int64_t v_stride, const void* wq, const void* wk, const void* wv, int K,
+                                    void* tail, const int* cu, const int* slot, const int* reset, int S,
+                                    const int* row_start, const int* row_slot, const int* positions,
+                                    const float* cos_sin, int rot_dim, int unit_norm, float eps, void* q_out,
+                                    void* k_cache, void* v_cache, const int* slots, int T, int Hq, int Hkv, int dim,
+                                    int vdim, int D, int P, int f32, hipStream_t stream) {
+  if (T <= 0 || S <= 0) return 0;
+  const int esz = f32 ? 4 : 2;
+  auto al = [&](const void* p, int64_t stride) { return (((uintptr_t)p | (uintptr_t)(stride * esz)) & 15) == 0; };
+  if (K < 0 || K > CV_MAXK || dim % 8 || vdim % 8 || dim > D || vdim > D || (D != 64 && D != 128 && D != 256) ||
+      (rot_dim & 1) || rot_dim > dim || !al(q, q_stride) || !al(k, k_stride) || !al(v, v_stride) || !al(wq, 0) ||
+      !al(wk, 0) || !al(wv, 0) || !al(tail, 0) || !al(q_out, 0) || !al(k_cache, 0) ||
+      (((int64_t)(Hq + Hkv) * dim + (int64_t)Hkv * vdim) * esz) % 16)
+    return -9;
+  if (K > 1 && tail == nullptr) return -2;
+  const int gs = D / 8;
+  const int64_t items = (int64_t)T * (Hq + 2 * Hkv);
+  const unsigned grid = (unsigned)((items + 256 / gs - 1) / (256 / gs));
+#define CV_ARGS(TT)                                                                                                 \
+  (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v, v_stride, (const TT*)wq, (const TT*)wk,            \
+      (const TT*)wv, (const TT*)tail, row_start, row_slot, positions, cos_sin, rot_dim, unit_norm, eps, (TT*)q_out, \
+      (TT*)k_cache, (TT*)v_cache, slots, T, Hq, Hkv, dim, vdim, P
+#define CV_GS(TT, KK)                                                                                   \
+  do {                                                                                                  \
+    if (gs == 8) conv_rope_cache_vec_kernel<TT, KK, 8><<<grid, 256, 0, stream>>>(CV_ARGS(TT));          \
+    else if (gs == 16) conv_rope_cache_vec_kernel<TT, KK, 16><<<grid, 256, 0, stream>>>(CV_ARGS(TT));   \
+    else conv_rope_cache_vec_kernel<TT, KK, 32><<<grid, 256, 0, stream>>>(CV_ARGS(TT));                 \
+  } while (0)
+#define CV_K(TT)                     \
+  switch (K) {                       \
+    case 0: CV_GS(TT, 0); break;     \
+    case 1: CV_GS(TT, 1); break;     \
+    case 2: CV_GS(TT, 2); break;     \
+    case 3: CV_GS(TT, 3); break;     \
+    case 4: CV_GS(TT, 4); break;     \
+    case 5: CV_GS(TT, 5); break;     \
+    default: CV_GS(TT, 6); break;    \
+  }
+  if (f32) { CV_K(float) } else { CV_K(bf16) }
+#undef CV_K
+#undef CV_GS
+#undef CV_ARGS
+  OME_CHECK_LAUNCH();
+  if (K > 1) {
+    const int C = (Hq + Hkv) * dim + Hkv * vdim;
+    const dim3 g2((C + 255) / 256, S);
+    if (S > 65535) return -3;
+    if (f32)
+      conv_tail_kernel<float><<<g2, 256, 0, stream>>>((const float*)q, q_stride, (const float*)k, k_stride,
+                                                      (const float*)v, v_stride, (float*)tail, cu, slot, reset, K - 1,
+                                                      Hq * dim, Hkv * dim, C);
+    else
+      conv_tail_kernel<bf16><<<g2, 256, 0, stream>>>((const bf16*)q, q_stride, (const bf16*)k, k_stride,
+                                                     (const bf16*)v, v_stride, (bf16*)tail, cu, slot, reset, K - 1,
+                                                     Hq * dim, Hkv * dim, C);
+    OME_CHECK_LAUNCH();
+  }
+  return 0;
+}
+
 OME_API int ome_conv_rope_cache(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                                 int64_t v_stride, const void* wq, const void* wk, const void* wv, int K, void* tail,
                                 const int* cu, const int* slot, const int* reset, int S, const int* positions,

@@ -448,9 +448,11 @@ def kernel_table_milenex(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
         tail = torch.zeros(len(lens), 3, C, device=dev, dtype=bf)
         hn = torch.ones(D, device=dev, dtype=bf)
         nb = R * C * 2 * 2
+        srows = ops.seq_rows(sq, R)      # (once per step in the model, shared by its layers)
+        qv, kv_, vv = qkv[:, :Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D:]
         pair(f"conv_rope_cache 4 taps ({tag})",
-             lambda: ops.conv_rope_cache(qkv[:, :Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D], qkv[:, (Hq + Hkv) * D:], *cw, tail,
-                                         sq, pos, cs, 64, True, True, 1e-6, qo, kc, vc, slots, Hq, Hkv, D, D),
+             lambda: ops.conv_rope_cache(qv, kv_, vv, *cw, tail, sq, pos, cs, 64, True, True, 1e-6, qo, kc, vc, slots,
+                                         Hq, Hkv, D, D, rows=srows),
              lambda: ops.rope_qkv_cache(qkv, pos, cs, 64, qo, kc, vc, slots, Hq, Hkv, D, True, hn, hn, 1e-6), nb, nb,
              "like: Qwen3's per-head norm + rotary + cache write (no convolution)")
         # ---- clamped GLU with the shared expert's per-row gate vs without

@@ -28,7 +28,7 @@ framework's GEMM dispatch (``quant.linear``); everything between them is one of 
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import torch
 
@@ -46,6 +46,7 @@ class MixerCtx:
     meta: AttnMeta
     kv: PagedKVCache
     seqs: tuple
+    cache: dict = field(default_factory=dict)   # tensors derived once per step and shared by the layers
 
 
 def paged_attention(q: torch.Tensor, k_cache, v_cache, meta: AttnMeta, scale: float, window: int = -1,
@@ -583,9 +584,12 @@ class ConvRotaryAttention(_Block):
         p = linear(h, self.w_in)                                   # [T, q | k | v]
         q = torch.empty(T, self.Hq, self.D, dtype=h.dtype, device=h.device)
         k_cache, v_cache = ctx.kv.layer(self.layer)
+        rows = ctx.cache.get("rows")
+        if rows is None and h.is_cuda:
+            rows = ctx.cache["rows"] = ops.seq_rows(ctx.seqs, T)
         ops.conv_rope_cache(p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:], self.cq, self.ck, self.cv, self.tail, ctx.seqs,
                             ctx.meta.positions, self.cos_sin, self.rot_dims, self.interleaved, self.unit_norm, self.eps,
-                            q, k_cache, v_cache, ctx.meta.slots, self.Hq, self.Hkv, self.dim, self.vdim)
+                            q, k_cache, v_cache, ctx.meta.slots, self.Hq, self.Hkv, self.dim, self.vdim, rows=rows)
         a = paged_attention(q, k_cache, v_cache, ctx.meta, self.scale, self.window, 0, self.sink)
         if self.D != self.vdim:
             a = a[:, :, :self.vdim].reshape(T, self.Hq * self.vdim)

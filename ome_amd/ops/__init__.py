@@ -11,7 +11,7 @@ import torch
 import torch.nn.functional as F
 
 from . import reference as ref
-from ._native import NativeError, available, call, ptr, stream_ptr  # noqa: F401
+from ._native import NativeError, available, call, load, ptr, stream_ptr  # noqa: F401
 
 
 def _gpu(t: torch.Tensor) -> bool:
@@ -1948,9 +1948,20 @@ def shift_norm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor 
     return new, out
 
 
+def seq_rows(seqs: tuple, T: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per row of a step: (first row of its sequence in the step, its state slot with bit 30 set
+    when the sequence starts in this step) -- what row-parallel kernels of stateful mixers read
+    instead of walking ``cu``.  One small computation per step, shared by all layers."""
+    cu, slot, reset = seqs
+    S = slot.shape[0]
+    r = torch.arange(T, dtype=torch.int64, device=cu.device)
+    seq = torch.bucketize(r, cu[1:S + 1].long(), right=True).clamp_(max=S - 1)
+    return cu[seq].contiguous(), (slot[seq] | (reset[seq] << 30)).to(torch.int32).contiguous()
+
+
 def conv_rope_cache(q, k, v, wq, wk, wv, tail, seqs, positions, cos_sin, rot_dim: int, interleaved: bool,
                     unit_norm: bool, eps: float, q_out, k_cache, v_cache, slots, Hq: int, Hkv: int, dim: int,
-                    vdim: int) -> None:
+                    vdim: int, rows: tuple | None = None) -> None:
     """Attention input with short causal convolutions.  q [T, Hq*dim], k [T, Hkv*dim], v [T,
     Hkv*vdim] (row-strided views of one projection) each pass a depthwise convolution over time
     (taps ``wq`` / ``wk`` / ``wv`` [channels, K], no bias, no activation; all None: no
@@ -1960,7 +1971,11 @@ def conv_rope_cache(q, k, v, wq, wk, wv, tail, seqs, positions, cos_sin, rot_dim
     its root mean square over ``dim`` AFTER the rotation (no weight).  q goes to ``q_out`` [T, Hq,
     D], k / v into the paged cache at ``slots`` (head tails beyond dim / vdim are zero).  ``tail``
     [slots, K-1, C] (C = all q, k, v channels, model dtype) keeps every sequence's last K-1
-    projected rows; ``seqs`` = (cu, slot, reset).  Convolution, rotation and norm are fp32."""
+    projected rows; ``seqs`` = (cu, slot, reset).  Convolution, rotation and norm are fp32.
+    ``rows`` = :func:`seq_rows` of the step (computed here when absent).  Head widths in multiples
+    of 8 with up to 6 taps and interleaved pairs run a row-parallel kernel without LDS (8 channels
+    per lane, 16-byte accesses, the tails rewritten by a second small launch); everything else the
+    tiled general kernel."""
     P, D = k_cache.shape[2], k_cache.shape[3]
     assert dim <= D and vdim <= D and rot_dim <= dim and rot_dim % 2 == 0
     if not _gpu(q):
@@ -1976,6 +1991,18 @@ def conv_rope_cache(q, k, v, wq, wk, wv, tail, seqs, positions, cos_sin, rot_dim
         assert tuple(wq.shape) == (Hq * dim, K) and tuple(wk.shape) == (Hkv * dim, K) and \
             tuple(wv.shape) == (Hkv * vdim, K) and wq.is_contiguous() and wk.is_contiguous() and wv.is_contiguous()
         assert K == 1 or (tail.is_contiguous() and tuple(tail.shape[1:]) == (K - 1, (Hq + Hkv) * dim + Hkv * vdim))
+    if (interleaved or rot_dim == 0) and K <= 6 and dim % 8 == 0 and vdim % 8 == 0:
+        rs, rl = rows if rows is not None else seq_rows(seqs, q.shape[0])
+        rc = load().ome_conv_rope_cache_vec(
+            q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), ptr(wq), ptr(wk), ptr(wv),
+            K, ptr(tail) if K > 1 else None, _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(),
+            slot.shape[0], _i32(rs).data_ptr(), _i32(rl).data_ptr(), _i32(positions).data_ptr(), cos_sin.data_ptr(),
+            int(rot_dim), int(bool(unit_norm)), float(eps), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            _i32(slots).data_ptr(), q.shape[0], Hq, Hkv, dim, vdim, D, P, f32, stream_ptr())
+        if rc == 0:
+            return
+        if rc != -9:     # -9: a shape or alignment the row-parallel kernel is not built for
+            raise NativeError(f"ome_conv_rope_cache_vec failed with code {rc}")
     call("ome_conv_rope_cache", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
          ptr(wq), ptr(wk), ptr(wv), K, ptr(tail) if K > 1 else None, _i32(cu).data_ptr(), _i32(slot).data_ptr(),
          _i32(reset).data_ptr(), slot.shape[0], _i32(positions).data_ptr(), cos_sin.data_ptr(), int(rot_dim),

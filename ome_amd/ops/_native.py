@@ -62,6 +62,8 @@ _SIGNATURES = {
                            i32, f32, i32, vp],
         "ome_conv_rope_cache": [vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32,
                                 f32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "ome_conv_rope_cache_vec": [vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, vp, vp, vp, vp, i32, vp, vp, vp, vp, i32,
+                                    i32, f32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "ome_talking_prefill": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i32, i32, vp, i64, vp, i64, i32, i32, i32, i32,
                                 i32, f32, i32, vp, vp, vp, vp, i32, i32, vp, vp, vp],
         "ome_talking_attn": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i64, vp, i64, i32, i32, i32, i32, i32, i32, f32,

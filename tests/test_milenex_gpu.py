@@ -38,7 +38,9 @@ def test_shift_norm_kernel(dt, W):
 @pytest.mark.parametrize("Hq,Hkv,dim,vdim,K,rot,il", [(4, 2, 8, 6, 3, 4, True), (3, 3, 10, 4, 2, 10, True),
                                                       (4, 1, 70, 36, 5, 6, False), (1, 1, 8, 8, 0, 8, True),
                                                       (32, 8, 128, 128, 4, 64, True), (2, 1, 200, 256, 33, 0, True),
-                                                      (6, 2, 96, 64, 1, 96, False)])
+                                                      (6, 2, 96, 64, 1, 96, False), (4, 2, 16, 24, 3, 8, True),
+                                                      (2, 2, 72, 40, 2, 72, True), (8, 2, 128, 128, 5, 64, True),
+                                                      (2, 1, 256, 256, 6, 128, True), (3, 1, 64, 64, 1, 0, True)])
 def test_conv_rope_cache_kernel(dt, Hq, Hkv, dim, vdim, K, rot, il):
     """Three sequences in one batch (a continued one, a fresh one on a dirty slot, a single row),
     two steps, against the reference op; caches and tails compared too."""
