@@ -468,8 +468,9 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
     const int pA = bt[kb / P];
     const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
     // the value fragments of this tile are asked for now and used in (c), two barriers later
-    bf16x8 vpre[NB];
-    if (uni) {
+    constexpr bool VPRE = HPW * D <= 256;   // (with 4 heads x 128 dims the accumulators leave no registers for it)
+    bf16x8 vpre[VPRE ? NB : 1];
+    if (VPRE && uni) {
       const bf16* vA = v_cache + pA * kpage + (int64_t)kv0 * D * P;
       const bf16* vB = v_cache + pB * kpage + (int64_t)kv0 * D * P;
 #pragma unroll
@@ -541,9 +542,11 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
         const int dim = 16 * nb + n;
         bf16x8 va;
         int kv_prev = -1;
-        if (uni) {
-          va = vpre[nb];
-          kv_prev = kv0;
+        if constexpr (VPRE) {
+          if (uni) {
+            va = vpre[nb];
+            kv_prev = kv0;
+          }
         }
 #pragma unroll
         for (int j = 0; j < HPW; ++j) {
@@ -605,7 +608,8 @@ __global__ __launch_bounds__(256) void talking_combine_kernel(const float* __res
                                                               int64_t gate_stride, bf16* __restrict__ out,
                                                               int64_t out_stride) {
   const int64_t b = blockIdx.x;
-  for (int o = threadIdx.x; o < H * vdim; o += 256) {
+  const int o = blockIdx.y * 256 + threadIdx.x;   // one output element per thread
+  if (o < H * vdim) {
     const int h = o / vdim, d = o - h * vdim;
     float a = 0.f;
     for (int z = 0; z < Z; ++z) a += part_o[(((b * Z + z) * H + h)) * D + d];
@@ -655,7 +659,7 @@ OME_API int ome_talking_prefill(const void* q, int64_t q_stride, const void* k_c
             (const bf16*)q, q_stride, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, bt_stride, cu_q,     \
             kv_lens, (const int2*)items, (const bf16*)gate, gate_stride, (bf16*)out, out_stride, H, Hkv, vdim, mul,  \
             window, sinks, r1, r2, talk, md, chunk, 1, part_ml, part_o);                                             \
-      talking_combine_kernel<<<n_items, 256, 0, stream>>>(part_o, splits, H, DD, vdim, (const bf16*)gate,            \
+      talking_combine_kernel<<<dim3(n_items, (H * vdim + 255) / 256), 256, 0, stream>>>(part_o, splits, H, DD, vdim, (const bf16*)gate,            \
                                                           gate_stride, (bf16*)out, out_stride);                      \
     } else {                                                                                                         \
       talking_prefill_kernel<DD, HH><<<grid, 64 * NW, lds, stream>>>(                                                \
