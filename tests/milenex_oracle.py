@@ -226,7 +226,7 @@ def rotary_layer(heads=4, kv_heads=2, dim=8, vdim=6, window=7, conv=3, rot_dims=
     return {"type": "attention", "mixer": m, "mlp": mlp}
 
 
-def biased_layer(heads=6, kv_heads=3, dim=6, vdim=10, window=9, scale=0.6, mlp=None):
+def biased_layer(heads=6, kv_heads=2, dim=6, vdim=10, window=9, scale=0.6, mlp=None):
     m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "mask": {"size": window}, "scale": scale}
     return {"type": "attention_2", "mixer": m, "mlp": mlp}
 
@@ -235,7 +235,7 @@ def dense(ff):
     return {"kind": "dense", "ff": ff}
 
 
-def moe(experts, top, ff, shared_ff, groups=1, keep=1, limit=1.5, shared_limit=1.0):
+def moe(experts, top, ff, shared_ff, groups=1, keep=1, limit=1.25, shared_limit=0.75):
     f = {"kind": "moe", "expert": {"ff": ff, "limit": limit},
          "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}}}
     if shared_ff:

@@ -86,7 +86,7 @@ def test_conv_rope_cache_kernel(dt, Hq, Hkv, dim, vdim, K, rot, il):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("H,Hkv,D,vdim,window,ctx", [(6, 3, 64, 64, 9, 40), (4, 1, 64, 7, 6, 33), (1, 1, 64, 64, 0, 50),
+@pytest.mark.parametrize("H,Hkv,D,vdim,window,ctx", [(6, 2, 64, 40, 9, 40), (4, 1, 64, 7, 6, 33), (1, 1, 64, 64, 0, 50),
                                                      (32, 8, 128, 128, 1024, 1500), (16, 1, 256, 200, 700, 900),
                                                      (18, 9, 64, 2, 20, 45), (32, 2, 128, 128, 0, 2100)])
 def test_talking_attn_kernel(dt, H, Hkv, D, vdim, window, ctx):
@@ -117,7 +117,7 @@ def test_talking_attn_kernel(dt, H, Hkv, D, vdim, window, ctx):
     _close(got, want, dt, want.float().abs().max().item())
 
 
-@pytest.mark.parametrize("H,Hkv,D,vdim,window", [(6, 3, 64, 64, 9), (4, 1, 64, 7, 6), (32, 8, 128, 128, 100),
+@pytest.mark.parametrize("H,Hkv,D,vdim,window", [(6, 2, 64, 40, 9), (4, 1, 64, 7, 6), (32, 8, 128, 128, 100),
                                                  (16, 2, 256, 200, 0), (1, 1, 64, 64, 40), (18, 9, 64, 2, 20),
                                                  (12, 4, 128, 96, 33)])
 def test_talking_prefill_kernel(H, Hkv, D, vdim, window):
@@ -158,7 +158,7 @@ def test_talking_prefill_kernel(H, Hkv, D, vdim, window):
     _close(got, want, BF, want.float().abs().max().item())
 
 
-@pytest.mark.parametrize("H,Hkv,D,vdim,window,ctx,B", [(6, 3, 64, 64, 136, 400, 4), (32, 8, 128, 128, 1024, 2100, 3),
+@pytest.mark.parametrize("H,Hkv,D,vdim,window,ctx,B", [(6, 2, 64, 40, 150, 400, 4), (32, 8, 128, 128, 1024, 2100, 3),
                                                        (4, 1, 64, 7, 6, 33, 2), (16, 2, 256, 200, 0, 700, 5),
                                                        (12, 4, 128, 96, 0, 90, 70), (1, 1, 64, 64, 40, 50, 300)])
 def test_talking_decode_kernel(H, Hkv, D, vdim, window, ctx, B):
