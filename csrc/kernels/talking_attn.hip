@@ -464,23 +464,19 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
   for (int j = 0; j < HPW; ++j)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) o[j][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // When all heads of the wave share one kv head (uni), its loads run ahead of their use: the key
+  // fragments of the NEXT tile are asked for right after (a) has used this tile's (same registers,
+  // in flight during (b) and (c)), the value fragments of this tile right after the first barrier (in
+  // flight during the mix).  Otherwise fragments are loaded where they are used, per kv head.
+  constexpr bool VPRE = HPW * D <= 256;   // (4 heads x 128 dims of accumulators leave no registers for the values)
+  bf16x8 ka[KS], kb8[KS];
+  if (uni && kv_lo < kv_end) load_k(kv_lo, kv0, ka, kb8);
   for (int kb = kv_lo; kb < kv_end; kb += 32) {
     const int pA = bt[kb / P];
     const int pB = (kb + P < kv_len) ? bt[kb / P + 1] : pA;
-    // the value fragments of this tile are asked for now and used in (c), two barriers later
-    constexpr bool VPRE = HPW * D <= 256;   // (with 4 heads x 128 dims the accumulators leave no registers for it)
-    bf16x8 vpre[VPRE ? NB : 1];
-    if (VPRE && uni) {
-      const bf16* vA = v_cache + pA * kpage + (int64_t)kv0 * D * P;
-      const bf16* vB = v_cache + pB * kpage + (int64_t)kv0 * D * P;
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        vpre[nb] = ta_cat44(ld4(vA + (16 * nb + n) * P + 4 * g), ld4(vB + (16 * nb + n) * P + 4 * g));
-    }
     // (a) final weights of this wave's heads
     {
-      bf16x8 ka[KS], kb8[KS];
-      int kv_prev = -1;
+      int kv_prev = uni ? kv0 : -1;
 #pragma unroll
       for (int j = 0; j < HPW; ++j) {
         const int head = wave * HPW + j;
@@ -513,7 +509,16 @@ __global__ __launch_bounds__(512) void talking_prefill_kernel(
         }
       }
     }
+    if (uni && kb + 32 < kv_end) load_k(kb + 32, kv0, ka, kb8);   // the next tile's keys
     __syncthreads();
+    bf16x8 vpre[VPRE ? NB : 1];
+    if (VPRE && uni) {
+      const bf16* vA = v_cache + pA * kpage + (int64_t)kv0 * D * P;
+      const bf16* vB = v_cache + pB * kpage + (int64_t)kv0 * D * P;
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        vpre[nb] = ta_cat44(ld4(vA + (16 * nb + n) * P + 4 * g), ld4(vB + (16 * nb + n) * P + 4 * g));
+    }
     // (b) mix over heads: one key slot (16 rows) per product column block
     for (int t = wave; t < 32; t += NW) {
       for (int mt = 0; mt < HM / 16; ++mt) {
