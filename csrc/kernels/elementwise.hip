@@ -327,6 +327,100 @@ OME_API int ome_embedding_f32(const int* ids, const void* table, float* out, int
   return 0;
 }
 
+// fp32 rows table[id] * scale + pair[r] with a hashed token-pair row r = (previous id * mul_prev +
+// id * mul_cur) mod buckets; a sequence's first token takes row `buckets` (the table's last).  The
+// id before a chunk's first row is state[slot] (one int per request slot); the workgroup of that row
+// reads it, then stores the chunk's last id there (no other workgroup touches the slot's entry).
+// Rows of sequence s are cu[s] .. cu[s+1]-1; reset[s] != 0: the sequence starts in this step.
+template <typename T>
+__global__ __launch_bounds__(256) void pair_embedding_f32_kernel(
+    const int* __restrict__ ids, const T* __restrict__ table, const T* __restrict__ pair, float* __restrict__ out,
+    int* __restrict__ state, int H, int V, float scale, int buckets, long long mul_prev, long long mul_cur,
+    const int* __restrict__ cu, const int* __restrict__ slot, const int* __restrict__ reset, int S) {
+  const int64_t t = blockIdx.x;
+  int s = 0;
+  while (s + 1 < S && cu[s + 1] <= (int)t) ++s;   // the sequence with cu[s] <= t < cu[s + 1]
+  const bool head = (int)t == cu[s];
+  const int id = ids[t];
+  const bool first = head && reset[s] != 0;
+  const int prev = head ? (first ? 0 : state[slot[s]]) : ids[t - 1];
+  long long r = ((long long)prev * mul_prev + (long long)id * mul_cur) % (long long)buckets;
+  if (r < 0) r += buckets;
+  if (first) r = buckets;
+  const bool ok = id >= 0 && id < V;
+  const T* row = table + (int64_t)(ok ? id : 0) * H;
+  const T* prow = pair + r * H;
+  for (int i = threadIdx.x; i < H; i += 256) out[t * H + i] = ok ? (float)row[i] * scale + (float)prow[i] : 0.f;
+  if (head) {
+    __syncthreads();   // every thread has read the old entry
+    if (threadIdx.x == 0) state[slot[s]] = ids[cu[s + 1] - 1];
+  }
+}
+
+OME_API int ome_pair_embedding_f32(const int* ids, const void* table, const void* pair, float* out, int* state, int T,
+                                   int H, int V, float scale, int buckets, int64_t mul_prev, int64_t mul_cur,
+                                   const int* cu, const int* slot, const int* reset, int S, int f32,
+                                   hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (buckets <= 0 || S <= 0) return -2;
+  if (f32)
+    pair_embedding_f32_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, (const float*)pair, out, state, H,
+                                                            V, scale, buckets, mul_prev, mul_cur, cu, slot, reset, S);
+  else
+    pair_embedding_f32_kernel<bf16><<<T, 256, 0, stream>>>(ids, (const bf16*)table, (const bf16*)pair, out, state, H,
+                                                           V, scale, buckets, mul_prev, mul_cur, cu, slot, reset, S);
+  OME_CHECK_LAUNCH();
+  return 0;
+}
+
+// Combine of a two-map (differential) attention.  a [T, 2 H, D]: per kv group g of R query heads,
+// first the R outputs of map 1, then the R outputs of map 2 (head h = g R + r: a1 = a[(2 g) R + r],
+// a2 = a[(2 g + 1) R + r]).  out[t, h, :] = o / sqrt(mean(o^2) + eps) * out_scale with o = a1 - lam a2
+// over the first vdim <= D columns (fp32, one rounding); out is contiguous [T, H * vdim].  One wave
+// per (row, head), vdim <= 64 * DN_MAX.
+constexpr int DN_MAX = 4;
+template <typename T>
+__global__ __launch_bounds__(256) void diff_head_norm_kernel(const T* __restrict__ a, T* __restrict__ out, int H, int R,
+                                                             int D, int vdim, float lam, float eps, float out_scale) {
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int h = blockIdx.y * 4 + wave; h < H; h += 4 * gridDim.y) {
+    const int g = h / R, r = h - g * R;
+    const T* a1 = a + (t * 2 * H + (int64_t)(2 * g) * R + r) * D;
+    const T* a2 = a1 + (int64_t)R * D;
+    float o[DN_MAX];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < DN_MAX; ++k) {
+      const int d = lane + 64 * k;
+      o[k] = d < vdim ? (float)a1[d] - lam * (float)a2[d] : 0.f;
+      ss += o[k] * o[k];
+    }
+    const float rs = out_scale / sqrtf(wave_sum(ss) / (float)vdim + eps);
+    T* op = out + (t * H + h) * vdim;
+#pragma unroll
+    for (int k = 0; k < DN_MAX; ++k) {
+      const int d = lane + 64 * k;
+      if (d < vdim) op[d] = (T)(o[k] * rs);
+    }
+  }
+}
+
+OME_API int ome_diff_head_norm(const void* a, void* out, int T, int H, int R, int D, int vdim, float lam, float eps,
+                               float out_scale, int f32, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H <= 0 || R <= 0 || H % R || vdim <= 0 || vdim > D || vdim > 64 * DN_MAX) return -2;
+  const dim3 grid(T, T >= 1024 ? 1 : (H + 3) / 4);
+  if (f32)
+    diff_head_norm_kernel<float><<<grid, 256, 0, stream>>>((const float*)a, (float*)out, H, R, D, vdim, lam, eps,
+                                                           out_scale);
+  else
+    diff_head_norm_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)a, (bf16*)out, H, R, D, vdim, lam, eps,
+                                                          out_scale);
+  OME_CHECK_LAUNCH();
+  return 0;
+}
+
 // Output gate of an attention layer: out[t, h * vdim + d] = o[t, h, d] * gate(g[t, h * vdim + d]),
 // d < vdim <= D (o's head rows are D wide; the padding beyond vdim is dropped).  kind 0: sigmoid,
 // 1: SiLU.

@@ -55,17 +55,20 @@ __global__ __launch_bounds__(256) void mla_attn_kernel(
     const bf16* __restrict__ q, int64_t q_stride_t, const bf16* __restrict__ cache,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_row,
     const int* __restrict__ kv_lens, int H, float scale_log2, int parts, bf16* __restrict__ out,
-    int64_t out_stride_t, float* __restrict__ ws_o, float* __restrict__ ws_ml, const float* __restrict__ sinks) {
+    int64_t out_stride_t, float* __restrict__ ws_o, float* __restrict__ ws_ml, const float* __restrict__ sinks,
+    int window) {
   constexpr int CH = DK / 8, NB = DV / 64, NST = (KT * CH + 255) / 256;   // NB 16-dim blocks per wave
   __shared__ __attribute__((aligned(16))) bf16 sK[KT * lds_chunks<DK>() * 8];
   const int t = blockIdx.x, h0 = blockIdx.y * 16, part = blockIdx.z;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int col = lane & 15, g = lane >> 4;
   const int L = kv_lens[t];
+  const int lo = window > 0 ? max(L - window, 0) : 0;   // sliding window: keys [lo, L) only
   const int n_pages = (L + 15) >> 4;
   const int pairs = (n_pages + 1) >> 1;
-  const int per_part = (pairs + parts - 1) / parts;
-  const int pair_begin = part * per_part, pair_end = min(pairs, pair_begin + per_part);
+  const int pair_lo = lo / KT;                          // key tiles wholly before the window are skipped
+  const int per_part = (pairs - pair_lo + parts - 1) / parts;
+  const int pair_begin = pair_lo + part * per_part, pair_end = min(pairs, pair_begin + per_part);
   const int* bt = block_tables + (int64_t)tok_row[t] * bt_stride;
   const int64_t ws_row = ((int64_t)t * H + h0 + col) * parts + part;
 
@@ -123,8 +126,9 @@ __global__ __launch_bounds__(256) void mla_attn_kernel(
     float mx = OME_NEG_INF;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      s0[i] = (kbase + 4 * g + i < L) ? s0[i] * scale_log2 : OME_NEG_INF;
-      s1[i] = (kbase + 16 + 4 * g + i < L) ? s1[i] * scale_log2 : OME_NEG_INF;
+      const int k0 = kbase + 4 * g + i, k1 = k0 + 16;
+      s0[i] = (k0 < L && k0 >= lo) ? s0[i] * scale_log2 : OME_NEG_INF;
+      s1[i] = (k1 < L && k1 >= lo) ? s1[i] * scale_log2 : OME_NEG_INF;
       mx = fmaxf(mx, fmaxf(s0[i], s1[i]));
     }
     mx = group4_max(mx);
@@ -410,7 +414,7 @@ template <int DK, int DV>
 static void mla_launch(const void* q, int64_t q_stride_t, const void* cache, const int* block_tables, int bt_stride,
                        const int* tok_row, const int* kv_lens, int T, int H, float scale_log2, int parts, void* out,
                        int64_t out_stride_t, float* ws_o, float* ws_ml, hipStream_t stream,
-                       const float* sinks = nullptr) {
+                       const float* sinks = nullptr, int window = -1) {
   // all-heads kernel when the heads tile into groups of 128 (DeepSeek-V3 / Kimi-K2 at TP 1) or 64
   // (TP 2): one latent stream per token and partition; else the 16-head kernel.  OME_MLA_ALL=0
   // forces the 16-head kernel (A/B timing).  Batches of at most OME_MLA_ALL_MIN_T tokens (default
@@ -422,8 +426,8 @@ static void mla_launch(const void* q, int64_t q_stride_t, const void* cache, con
   const bool all_ok = all_env && T > min_t;
   bool done = false;
   if constexpr (DK == 576) {
-    if (sinks != nullptr) {
-      // (the all-heads kernel has no sink term: sinks take the 16-head kernel)
+    if (sinks != nullptr || window > 0) {
+      // (the all-heads kernel has no sink term and no window: these take the 16-head kernel)
     } else if (all_ok && H % 128 == 0) {
       mla_attn_all_kernel<DK, DV, 8><<<dim3(T, H / 128, parts), 512, 0, stream>>>(
           (const bf16*)q, q_stride_t, (const bf16*)cache, block_tables, bt_stride, tok_row, kv_lens, H, scale_log2,
@@ -439,7 +443,7 @@ static void mla_launch(const void* q, int64_t q_stride_t, const void* cache, con
   if (!done)
     mla_attn_kernel<DK, DV><<<dim3(T, (H + 15) / 16, parts), 256, 0, stream>>>(
         (const bf16*)q, q_stride_t, (const bf16*)cache, block_tables, bt_stride, tok_row, kv_lens, H, scale_log2,
-        parts, (bf16*)out, out_stride_t, ws_o, ws_ml, sinks);
+        parts, (bf16*)out, out_stride_t, ws_o, ws_ml, sinks, window);
   if (parts > 1)
     mla_reduce_kernel<DV><<<dim3(T, H), DV / 4, 0, stream>>>(ws_o, ws_ml, H, parts, (bf16*)out, out_stride_t, sinks);
 }
@@ -466,19 +470,20 @@ OME_API int ome_mla_attn(const void* q, int64_t q_stride_t, const void* cache, c
 // Latent attention over rows of any latent / rotary width, padded to the kernel's tiling: a cache
 // row is [latent (dv_pad wide: the values, zero beyond the latent) | rotary key (dk - dv_pad wide,
 // zero beyond it)], dv_pad a multiple of 64 up to 256 or 512, dk - dv_pad 32 or 64.  The 16-head kernel
-// serves every step kind; sinks optional.  Zero columns add nothing to a score, and the output's
-// zero columns are dropped by the caller.
+// serves every step kind; sinks optional; window > 0: a token sees only the last `window` of its
+// kv_lens keys.  Zero columns add nothing to a score, and the output's zero columns are dropped by
+// the caller.
 OME_API int ome_latent_attn(const void* q, int64_t q_stride_t, const void* cache, const int* block_tables,
                             int bt_stride, const int* tok_row, const int* kv_lens, int T, int H, int dk, int dv,
                             float scale, int parts, void* out, int64_t out_stride_t, float* ws_o, float* ws_ml,
-                            const float* sinks, hipStream_t stream) {
+                            const float* sinks, int window, hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || parts < 1 || (parts > 1 && (!ws_o || !ws_ml))) return -2;
   const float scale_log2 = scale * 1.4426950408889634f;
 #define LATENT_CASE(DK_, DV_)                                                                                       \
   if (dk == DK_ && dv == DV_) {                                                                                     \
     mla_launch<DK_, DV_>(q, q_stride_t, cache, block_tables, bt_stride, tok_row, kv_lens, T, H, scale_log2, parts,  \
-                         out, out_stride_t, ws_o, ws_ml, stream, sinks);                                            \
+                         out, out_stride_t, ws_o, ws_ml, stream, sinks, window);                                    \
     OME_CHECK_LAUNCH();                                                                                             \
     return 0;                                                                                                       \
   }

@@ -33,7 +33,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
                                                         int E, int k, int renorm, int scoring,
                                                         const float* __restrict__ bias, int n_group, int topk_group,
                                                         int group_mode, float* __restrict__ topk_w,
-                                                        int* __restrict__ topk_ids) {
+                                                        int* __restrict__ topk_ids,
+                                                        const float* __restrict__ logit_bias) {
   __shared__ float s_key[4][512];
   __shared__ int s_gsel[4][64];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -46,8 +47,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
     const int e = lane + 64 * i;
-    v[i] = e < E ? (float)row[e] : OME_NEG_INF;
-    mx = fmaxf(mx, v[i]);
+    v[i] = e < E ? (float)row[e] + (logit_bias ? logit_bias[e] : 0.f) : OME_NEG_INF;   // (a bias of the logits
+    mx = fmaxf(mx, v[i]);                                                               // counts in the scores)
   }
   mx = wave_max(mx);
   float sum = 0.f;
@@ -167,17 +168,17 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
 
 OME_API int ome_moe_route(const void* logits, int is_bf16, int64_t stride, int n_tok, int E, int k, int renorm,
                           int scoring, const float* bias, int n_group, int topk_group, int group_mode,
-                          float* topk_w, int* topk_ids, hipStream_t stream) {
+                          float* topk_w, int* topk_ids, const float* logit_bias, hipStream_t stream) {
   if (n_tok <= 0) return 0;
   if (E > 512 || k > E || k <= 0) return -2;
   if (group_mode && n_group > 1 && (E % n_group || n_group > 64 || topk_group > n_group)) return -2;
   const int g = (n_tok + 3) / 4;
   if (is_bf16)
     moe_route_kernel<bf16><<<g, 256, 0, stream>>>((const bf16*)logits, stride, n_tok, E, k, renorm, scoring, bias,
-                                                  n_group, topk_group, group_mode, topk_w, topk_ids);
+                                                  n_group, topk_group, group_mode, topk_w, topk_ids, logit_bias);
   else
     moe_route_kernel<float><<<g, 256, 0, stream>>>((const float*)logits, stride, n_tok, E, k, renorm, scoring, bias,
-                                                   n_group, topk_group, group_mode, topk_w, topk_ids);
+                                                   n_group, topk_group, group_mode, topk_w, topk_ids, logit_bias);
   OME_CHECK_LAUNCH();
   return 0;
 }

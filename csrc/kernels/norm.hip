@@ -668,7 +668,8 @@ OME_API int ome_row_norm(const void* x, int64_t x_stride, int x_f32, const void*
 
 // ------------------------------------------------------------------------------------------
 // Pre-norm step of an fp32 residual stream with a token shift.  For row t of sequence s:
-//   v[t]   = res_in[t] + s1 * x1[t] + s2 * x2[t]            (either addend may be absent)
+//   v[t]   = res_in[t] + s1 * x1[t] + s2 * x2[t] + bias       (either addend may be absent; bias:
+//                                                            one row of width H for all rows, or null)
 //   n[t]   = v[t] / sqrt(mean(v[t]^2) + eps) * (w_off + w)  (fp32; w_off = 1 for weights stored
 //                                                            as the offset from one)
 //   out[t] = n[t] + (n[t-1] - n[t]) * mu                     (rounded once, to T)
@@ -682,22 +683,26 @@ OME_API int ome_row_norm(const void* x, int64_t x_stride, int x_f32, const void*
 namespace {
 template <typename T>
 __device__ __forceinline__ float shift_row_rs(const float* __restrict__ r, const T* __restrict__ a, float s1,
-                                              const T* __restrict__ b, float s2, int H, float eps, float* red) {
+                                              const T* __restrict__ b, float s2, const T* __restrict__ c, int H,
+                                              float eps, float* red) {
   float ss = 0.f;
   for (int i = threadIdx.x; i < H; i += 256) {
     float v = r[i];
     if (a != nullptr) v += s1 * (float)a[i];
     if (b != nullptr) v += s2 * (float)b[i];
+    if (c != nullptr) v += (float)c[i];
     ss += v * v;
   }
   return 1.f / sqrtf(block_sum<256>(ss, red) / (float)H + eps);
 }
 
 template <typename T>
-__device__ __forceinline__ float shift_val(const float* r, const T* a, float s1, const T* b, float s2, int i) {
+__device__ __forceinline__ float shift_val(const float* r, const T* a, float s1, const T* b, float s2, const T* c,
+                                           int i) {
   float v = r[i];
   if (a != nullptr) v += s1 * (float)a[i];
   if (b != nullptr) v += s2 * (float)b[i];
+  if (c != nullptr) v += (float)c[i];
   return v;
 }
 
@@ -707,18 +712,18 @@ __global__ __launch_bounds__(256) void shift_norm_kernel(
     int64_t x1_stride, float s1, const T* __restrict__ x2, int64_t x2_stride, float s2, const T* __restrict__ w,
     float w_off, const T* __restrict__ mu, float* __restrict__ state, const int* __restrict__ cu,
     const int* __restrict__ slot, const int* __restrict__ reset, int S, T* __restrict__ out, int64_t out_stride,
-    int H, float eps) {
+    int H, float eps, const T* __restrict__ bias) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const float* r = res_in + row * res_stride;
   const T* a = x1 != nullptr ? x1 + row * x1_stride : nullptr;
   const T* b = x2 != nullptr ? x2 + row * x2_stride : nullptr;
-  const float rs = shift_row_rs(r, a, s1, b, s2, H, eps, red);
+  const float rs = shift_row_rs(r, a, s1, b, s2, bias, H, eps, red);
   float* ro = res_out + row * res_stride;
   T* o = out + row * out_stride;
   if (mu == nullptr) {
     for (int i = threadIdx.x; i < H; i += 256) {
-      const float v = shift_val(r, a, s1, b, s2, i);
+      const float v = shift_val(r, a, s1, b, s2, bias, i);
       ro[i] = v;
       o[i] = (T)(v * rs * (w_off + (float)w[i]));
     }
@@ -731,10 +736,10 @@ __global__ __launch_bounds__(256) void shift_norm_kernel(
     const float* rp = r - res_stride;
     const T* ap = a != nullptr ? a - x1_stride : nullptr;
     const T* bp = b != nullptr ? b - x2_stride : nullptr;
-    const float rsp = shift_row_rs(rp, ap, s1, bp, s2, H, eps, red);
+    const float rsp = shift_row_rs(rp, ap, s1, bp, s2, bias, H, eps, red);
     for (int i = threadIdx.x; i < H; i += 256) {
-      const float v = shift_val(r, a, s1, b, s2, i), wi = w_off + (float)w[i];
-      const float n = v * rs * wi, np = shift_val(rp, ap, s1, bp, s2, i) * rsp * wi;
+      const float v = shift_val(r, a, s1, b, s2, bias, i), wi = w_off + (float)w[i];
+      const float n = v * rs * wi, np = shift_val(rp, ap, s1, bp, s2, bias, i) * rsp * wi;
       ro[i] = v;
       o[i] = (T)(n + (np - n) * (float)mu[i]);
     }
@@ -746,13 +751,13 @@ __global__ __launch_bounds__(256) void shift_norm_kernel(
   const float* rl = r + d * res_stride;
   const T* al = a != nullptr ? a + d * x1_stride : nullptr;
   const T* bl = b != nullptr ? b + d * x2_stride : nullptr;
-  const float rsl = d > 0 ? shift_row_rs(rl, al, s1, bl, s2, H, eps, red) : rs;
+  const float rsl = d > 0 ? shift_row_rs(rl, al, s1, bl, s2, bias, H, eps, red) : rs;
   for (int i = threadIdx.x; i < H; i += 256) {
-    const float v = shift_val(r, a, s1, b, s2, i), wi = w_off + (float)w[i];
+    const float v = shift_val(r, a, s1, b, s2, bias, i), wi = w_off + (float)w[i];
     const float n = v * rs * wi, np = fresh ? 0.f : st[i];
     ro[i] = v;
     o[i] = (T)(n + (np - n) * (float)mu[i]);
-    st[i] = d > 0 ? shift_val(rl, al, s1, bl, s2, i) * rsl * wi : n;
+    st[i] = d > 0 ? shift_val(rl, al, s1, bl, s2, bias, i) * rsl * wi : n;
   }
 }
 }  // namespace
@@ -779,11 +784,11 @@ __device__ __forceinline__ void sn_st4(T* p, f32x4 v) {
   }
 }
 
-// v = r + s1 a + s2 b of one row into registers; returns 1 / rms
+// v = r + s1 a + s2 b + c of one row into registers; returns 1 / rms
 template <typename T, int NCH>
 __device__ __forceinline__ float sn_row(const float* __restrict__ r, const T* __restrict__ a, float s1,
-                                        const T* __restrict__ b, float s2, int H, float eps, float* red,
-                                        f32x4 (&v)[NCH]) {
+                                        const T* __restrict__ b, float s2, const T* __restrict__ cb, int H, float eps,
+                                        float* red, f32x4 (&v)[NCH]) {
   float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < NCH; ++k) {
@@ -792,6 +797,7 @@ __device__ __forceinline__ float sn_row(const float* __restrict__ r, const T* __
       f32x4 x = *reinterpret_cast<const f32x4*>(r + c);
       if (a != nullptr) x += s1 * sn_ld4<T>(a + c);
       if (b != nullptr) x += s2 * sn_ld4<T>(b + c);
+      if (cb != nullptr) x += sn_ld4<T>(cb + c);
       v[k] = x;
       ss += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
     }
@@ -805,14 +811,14 @@ __global__ __launch_bounds__(256) void shift_norm_vec_kernel(
     int64_t x1_stride, float s1, const T* __restrict__ x2, int64_t x2_stride, float s2, const T* __restrict__ w,
     float w_off, const T* __restrict__ mu, float* __restrict__ state, const int* __restrict__ cu,
     const int* __restrict__ slot, const int* __restrict__ reset, int S, T* __restrict__ out, int64_t out_stride,
-    int H, float eps) {
+    int H, float eps, const T* __restrict__ bias) {
   __shared__ float red[4];
   const int64_t row = blockIdx.x;
   const float* r = res_in + row * res_stride;
   const T* a = x1 != nullptr ? x1 + row * x1_stride : nullptr;
   const T* b = x2 != nullptr ? x2 + row * x2_stride : nullptr;
   f32x4 v[NCH], p[NCH];
-  const float rs = sn_row<T, NCH>(r, a, s1, b, s2, H, eps, red, v);
+  const float rs = sn_row<T, NCH>(r, a, s1, b, s2, bias, H, eps, red, v);
   float* ro = res_out + row * res_stride;
   T* o = out + row * out_stride;
   // kind of row: 0 no shift, 1 the row before is in this step, 2 first row of its sequence
@@ -825,10 +831,10 @@ __global__ __launch_bounds__(256) void shift_norm_vec_kernel(
   }
   if (kind == 1) {
     rsp = sn_row<T, NCH>(r - res_stride, a != nullptr ? a - x1_stride : nullptr, s1,
-                         b != nullptr ? b - x2_stride : nullptr, s2, H, eps, red, p);
+                         b != nullptr ? b - x2_stride : nullptr, s2, bias, H, eps, red, p);
   } else if (kind == 2 && d > 0) {   // the sequence's last row of the step: the new state
     rsp = sn_row<T, NCH>(r + (int64_t)d * res_stride, a != nullptr ? a + (int64_t)d * x1_stride : nullptr, s1,
-                         b != nullptr ? b + (int64_t)d * x2_stride : nullptr, s2, H, eps, red, p);
+                         b != nullptr ? b + (int64_t)d * x2_stride : nullptr, s2, bias, H, eps, red, p);
   }
   float* st = kind == 2 ? state + (int64_t)slot[s] * H : nullptr;
   const bool fresh = kind == 2 && reset[s] != 0;
@@ -857,18 +863,20 @@ __global__ __launch_bounds__(256) void shift_norm_vec_kernel(
 OME_API int ome_shift_norm(const float* res_in, float* res_out, int64_t res_stride, const void* x1, int64_t x1_stride,
                            float s1, const void* x2, int64_t x2_stride, float s2, const void* w, float w_off,
                            const void* mu, float* state, const int* cu, const int* slot, const int* reset, int S,
-                           void* out, int64_t out_stride, int rows, int H, float eps, int f32, hipStream_t stream) {
+                           void* out, int64_t out_stride, int rows, int H, float eps, int f32, const void* bias,
+                           hipStream_t stream) {
   if (rows <= 0) return 0;
   if (H <= 0 || (mu != nullptr && (S <= 0 || state == nullptr))) return -2;
   const int esz = f32 ? 4 : 2;
   auto al = [](const void* p, int64_t stride, int e) { return (((uintptr_t)p | (uintptr_t)(stride * e)) & (4 * e - 1)) == 0; };
   if (H % 4 == 0 && H <= 8192 && al(res_in, res_stride, 4) && al(res_out, res_stride, 4) && al(x1, x1_stride, esz) &&
-      al(x2, x2_stride, esz) && al(w, 0, esz) && al(mu, 0, esz) && al(out, out_stride, esz) && al(state, H, 4)) {
+      al(x2, x2_stride, esz) && al(w, 0, esz) && al(mu, 0, esz) && al(out, out_stride, esz) && al(state, H, 4) &&
+      al(bias, 0, esz)) {
 #define SN_VEC(TT, N)                                                                                                \
   shift_norm_vec_kernel<TT, N><<<rows, 256, 0, stream>>>(res_in, res_out, res_stride, (const TT*)x1, x1_stride, s1,   \
                                                          (const TT*)x2, x2_stride, s2, (const TT*)w, w_off,           \
                                                          (const TT*)mu, state, cu, slot, reset, S, (TT*)out,          \
-                                                         out_stride, H, eps)
+                                                         out_stride, H, eps, (const TT*)bias)
 #define SN_PICK(TT)                 \
   do {                              \
     if (H <= 1024) SN_VEC(TT, 1);   \
@@ -887,12 +895,12 @@ OME_API int ome_shift_norm(const float* res_in, float* res_out, int64_t res_stri
     shift_norm_kernel<float><<<rows, 256, 0, stream>>>(res_in, res_out, res_stride, (const float*)x1, x1_stride, s1,
                                                        (const float*)x2, x2_stride, s2, (const float*)w, w_off,
                                                        (const float*)mu, state, cu, slot, reset, S, (float*)out,
-                                                       out_stride, H, eps);
+                                                       out_stride, H, eps, (const float*)bias);
   else
     shift_norm_kernel<bf16><<<rows, 256, 0, stream>>>(res_in, res_out, res_stride, (const bf16*)x1, x1_stride, s1,
                                                       (const bf16*)x2, x2_stride, s2, (const bf16*)w, w_off,
                                                       (const bf16*)mu, state, cu, slot, reset, S, (bf16*)out,
-                                                      out_stride, H, eps);
+                                                      out_stride, H, eps, (const bf16*)bias);
   OME_CHECK_LAUNCH();
   return 0;
 }

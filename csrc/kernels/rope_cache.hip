@@ -239,14 +239,18 @@ OME_API int ome_kv_cache_write(const void* k, const void* v, int64_t kv_stride, 
 // first rot_dim dims of every head are rotated (interleaved: dim 2i with 2i+1; else i with
 // i + rot_dim/2) by the angle row cos_sin[pos] = [cos(rot_dim/2) | sin(rot_dim/2)], all in fp32
 // with one rounding to bf16 at the store.  Heads are written D wide (q_out [T, Hq, D], K cache
-// [page, Hkv, P, D], V cache [page, Hkv, D, P]) with zeros beyond dim / vdim.
+// [page, Hkv, P, D], V cache [page, Hkv, D, P]) with zeros beyond dim / vdim.  q_scale (fp32 [Hq],
+// nullable): a per-head factor on the rotated query (a temperature), applied in fp32 before the
+// rounding.  v_rep > 1: v holds Hkv / v_rep heads and cache head h stores value head h / v_rep
+// (several key heads attending over the same values).
 template <typename T>
 __global__ __launch_bounds__(256) void wide_norm_rope_cache_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride,
     const T* __restrict__ v, int64_t v_stride, const int* __restrict__ positions,
     const float* __restrict__ cos_sin, int rot_dim, int interleaved, const T* __restrict__ qn_w,
     const T* __restrict__ kn_w, float eps, T* __restrict__ q_out, T* __restrict__ k_cache,
-    T* __restrict__ v_cache, const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P) {
+    T* __restrict__ v_cache, const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P,
+    const float* __restrict__ q_scale, int v_rep) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
   const T* qr = q + t * q_stride;
@@ -302,6 +306,10 @@ __global__ __launch_bounds__(256) void wide_norm_rope_cache_kernel(
     }
     if (is_q) {
       T* dst = q_out + (t * Hq + hh) * D;
+      if (q_scale != nullptr) {
+        a *= q_scale[hh];
+        b *= q_scale[hh];
+      }
       if (d0 < D) dst[d0] = (T)a;
       if (d1 < D) dst[d1] = (T)b;
     } else if (slot >= 0) {
@@ -314,7 +322,7 @@ __global__ __launch_bounds__(256) void wide_norm_rope_cache_kernel(
   if (slot >= 0) {
     for (int i = threadIdx.x; i < Hkv * D; i += 256) {
       const int kh = i / D, d = i - kh * D;
-      const float x = d < vdim ? (float)vr[kh * vdim + d] : 0.f;
+      const float x = d < vdim ? (float)vr[(kh / v_rep) * vdim + d] : 0.f;
       v_cache[((page * Hkv + kh) * D + d) * P + off] = (T)x;
     }
   }
@@ -329,7 +337,8 @@ __global__ __launch_bounds__(256) void wide_norm_rope_cache_vec_kernel(
     const bf16* __restrict__ v, int64_t v_stride, const int* __restrict__ positions,
     const float* __restrict__ cos_sin, int rot_dim, const bf16* __restrict__ qn_w, const bf16* __restrict__ kn_w,
     float eps, bf16* __restrict__ q_out, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
-    const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P) {
+    const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P,
+    const float* __restrict__ q_scale, int v_rep) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
   const bf16* qr = q + t * q_stride;
@@ -390,8 +399,9 @@ __global__ __launch_bounds__(256) void wide_norm_rope_cache_vec_kernel(
           f[2 * j + 1] = b * c + a * sn;
         }
       }
+      const float qs = is_q && q_scale != nullptr ? q_scale[hh] : 1.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = (bf16)f[j];
+      for (int j = 0; j < 8; ++j) o[j] = (bf16)(f[j] * qs);
     }
     if (is_q) st8(q_out + (t * Hq + hh) * D + d0, o);
     else st8(k_cache + ((page * Hkv + hh) * P + off) * D + d0, o);
@@ -399,7 +409,7 @@ __global__ __launch_bounds__(256) void wide_norm_rope_cache_vec_kernel(
   if (slot >= 0) {   // v: lanes take consecutive dims (rows 2 * P bytes apart), zeros beyond vdim
     for (int i = threadIdx.x; i < Hkv * D; i += 256) {
       const int kh = i / D, d = i - kh * D;
-      v_cache[((page * Hkv + kh) * D + d) * P + off] = d < vdim ? vr[kh * vdim + d] : (bf16)0.f;
+      v_cache[((page * Hkv + kh) * D + d) * P + off] = d < vdim ? vr[(kh / v_rep) * vdim + d] : (bf16)0.f;
     }
   }
 }
@@ -408,15 +418,17 @@ OME_API int ome_wide_norm_rope_cache(const void* q, int64_t q_stride, const void
                                      int64_t v_stride, const int* positions, const float* cos_sin, int rot_dim,
                                      int interleaved, const void* qn_w, const void* kn_w, float eps, void* q_out,
                                      void* k_cache, void* v_cache, const int* slots, int T, int Hq, int Hkv, int dim,
-                                     int vdim, int D, int P, int f32, hipStream_t stream) {
+                                     int vdim, int D, int P, int f32, const float* q_scale, int v_rep,
+                                     hipStream_t stream) {
   if (T <= 0) return 0;
   if (dim <= 0 || vdim <= 0 || dim > D || vdim > D || (D & 1) || rot_dim < 0 || rot_dim > dim || (rot_dim & 1))
     return -2;
+  if (v_rep < 1 || Hkv % v_rep) return -2;
   if (f32) {   // fp32 model: fp32 projections, norm weights, q and cache
     wide_norm_rope_cache_kernel<float><<<T, 256, 0, stream>>>(
         (const float*)q, q_stride, (const float*)k, k_stride, (const float*)v, v_stride, positions, cos_sin, rot_dim,
         interleaved, (const float*)qn_w, (const float*)kn_w, eps, (float*)q_out, (float*)k_cache, (float*)v_cache,
-        slots, Hq, Hkv, dim, vdim, D, P);
+        slots, Hq, Hkv, dim, vdim, D, P, q_scale, v_rep);
     OME_CHECK_LAUNCH();
     return 0;
   }
@@ -428,14 +440,14 @@ OME_API int ome_wide_norm_rope_cache(const void* q, int64_t q_stride, const void
     wide_norm_rope_cache_vec_kernel<<<T, 256, 0, stream>>>(
         (const bf16*)q, q_stride, (const bf16*)k, k_stride, (const bf16*)v, v_stride, positions, cos_sin, rot_dim,
         (const bf16*)qn_w, (const bf16*)kn_w, eps, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, slots, Hq, Hkv, dim,
-        vdim, D, P);
+        vdim, D, P, q_scale, v_rep);
     OME_CHECK_LAUNCH();
     return 0;
   }
   wide_norm_rope_cache_kernel<bf16><<<T, 256, 0, stream>>>(
       (const bf16*)q, q_stride, (const bf16*)k, k_stride, (const bf16*)v, v_stride, positions, cos_sin, rot_dim,
       interleaved, (const bf16*)qn_w, (const bf16*)kn_w, eps, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, slots,
-      Hq, Hkv, dim, vdim, D, P);
+      Hq, Hkv, dim, vdim, D, P, q_scale, v_rep);
   OME_CHECK_LAUNCH();
   return 0;
 }

@@ -440,7 +440,8 @@ OME_API int ome_gated_rmsnorm(const void* y, int64_t y_stride, const void* z, in
 }
 
 // ------------------------------------------------------------------------------------------
-// Residual causal convolution on an fp32 stream: out[r, c] = x[r, c] + sum_j w[c, j] * x[r - K + 1 + j, c]
+// Residual causal convolution: out[r, c] = x[r, c] + sum_j w[c, j] * x[r - K + 1 + j, c]; x is an
+// fp32 stream (TX = float) or a row already rounded to the taps' type (TX = T); sums are fp32
 // (tap K-1 on the current row, zeros before a sequence's start, no bias, no activation), over a
 // varlen batch; the last K-1 INPUT rows of every sequence live in `state` [slots, C, K-1] (fp32)
 // between steps.  Not recurrent, so time is parallel: grid (channel blocks, sequences, row tiles of
@@ -452,8 +453,8 @@ OME_API int ome_gated_rmsnorm(const void* y, int64_t y_stride, const void* z, in
 namespace {
 constexpr int CM_TILE = 64;
 
-template <typename T>
-__global__ __launch_bounds__(256) void conv_mix_kernel(const float* __restrict__ x, int64_t x_stride,
+template <typename T, typename TX>
+__global__ __launch_bounds__(256) void conv_mix_kernel(const TX* __restrict__ x, int64_t x_stride,
                                                        const T* __restrict__ w, T* __restrict__ out,
                                                        int64_t out_stride, float* __restrict__ state,
                                                        const int* __restrict__ cu, const int* __restrict__ slot,
@@ -473,13 +474,13 @@ __global__ __launch_bounds__(256) void conv_mix_kernel(const float* __restrict__
     const int L = r1 - r0;
     for (int j = 0; j < K - 1; ++j) {   // input index L - (K-1) + j of the chunk; negative = old tail
       const int i = L - (K - 1) + j;
-      st[j] = i >= 0 ? x[(int64_t)(r0 + i) * x_stride + c] : win[K - 1 + i];
+      st[j] = i >= 0 ? (float)x[(int64_t)(r0 + i) * x_stride + c] : win[K - 1 + i];
     }
   } else {
-    for (int j = 0; j < K - 1; ++j) win[j] = x[(int64_t)(a - (K - 1) + j) * x_stride + c];
+    for (int j = 0; j < K - 1; ++j) win[j] = (float)x[(int64_t)(a - (K - 1) + j) * x_stride + c];
   }
   for (int r = a; r < e; ++r) {
-    const float v = x[(int64_t)r * x_stride + c];
+    const float v = (float)x[(int64_t)r * x_stride + c];
     float acc = v + wt[K - 1] * v;
     for (int j = 0; j < K - 1; ++j) acc += wt[j] * win[j];
     for (int j = 0; j + 1 < K - 1; ++j) win[j] = win[j + 1];
@@ -489,20 +490,23 @@ __global__ __launch_bounds__(256) void conv_mix_kernel(const float* __restrict__
 }
 }  // namespace
 
-OME_API int ome_conv_mix(const float* x, int64_t x_stride, const void* w, void* out, int64_t out_stride, float* state,
+OME_API int ome_conv_mix(const void* x, int64_t x_stride, const void* w, void* out, int64_t out_stride, float* state,
                          const int* cu, const int* slot, const int* reset, int S, int T, int C, int K, int f32,
-                         hipStream_t stream) {
+                         int x_f32, hipStream_t stream) {
   if (S <= 0 || C <= 0 || T <= 0) return 0;
   if (K < 1 || K > 32) return -2;
   const int tiles = (T + CM_TILE - 1) / CM_TILE;
   if (tiles > 65535 || S > 65535) return -3;
   dim3 grid((C + 255) / 256, S, tiles);
   if (f32)
-    conv_mix_kernel<float><<<grid, 256, 0, stream>>>(x, x_stride, (const float*)w, (float*)out, out_stride, state, cu,
-                                                     slot, reset, C, K);
+    conv_mix_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, (const float*)w, (float*)out,
+                                                            out_stride, state, cu, slot, reset, C, K);
+  else if (x_f32)
+    conv_mix_kernel<bf16, float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, (const bf16*)w, (bf16*)out,
+                                                           out_stride, state, cu, slot, reset, C, K);
   else
-    conv_mix_kernel<bf16><<<grid, 256, 0, stream>>>(x, x_stride, (const bf16*)w, (bf16*)out, out_stride, state, cu,
-                                                    slot, reset, C, K);
+    conv_mix_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)x, x_stride, (const bf16*)w, (bf16*)out,
+                                                          out_stride, state, cu, slot, reset, C, K);
   OME_CHECK_LAUNCH();
   return 0;
 }

@@ -85,6 +85,10 @@ def model_class(cfg: ModelConfig):
         from ome_amd.models.metitar import MetitarForCausalLM
 
         return MetitarForCausalLM
+    if cfg.architecture == "Nivasun" or cfg.model_type == "nivasun":
+        from ome_amd.models.nivasun import NivasunForCausalLM
+
+        return NivasunForCausalLM
     if cfg.architecture == "Milenex" or cfg.model_type == "milenex":
         from ome_amd.models.milenex import MilenexForCausalLM
 
@@ -232,7 +236,7 @@ def supported(arch: str) -> bool:
         arch in ("JanusForConditionalGeneration", "MultiModalityCausalLM", "JanusMultiModalityCausalLM") or \
         arch in ("LlavaQwenForCausalLM", "LlavaOnevisionForConditionalGeneration") or \
         arch in ("BailingMoeForCausalLM", "XverseMoeForCausalLM", "Glm4vMoeForConditionalGeneration") or \
-        arch == "GptOssForCausalLM" or arch in ("Zavilorn", "Metitar", "Milenex") or arch in ("KimiVLForConditionalGeneration", "Kimi_K25ForConditionalGeneration") or \
+        arch == "GptOssForCausalLM" or arch in ("Zavilorn", "Metitar", "Milenex", "Nivasun") or arch in ("KimiVLForConditionalGeneration", "Kimi_K25ForConditionalGeneration") or \
         arch in ("Phi4MMForCausalLM", "Phi4MultimodalForCausalLM") or \
         arch in ("Grok1ModelForCausalLM", "Grok1ForCausalLM") or arch in ("TeleFLMModel", "TeleFLMForCausalLM") or \
         arch == "Phi3VForCausalLM" or arch in ("NemotronH_Nano_VL_V2", "NemotronVLForConditionalGeneration") or \

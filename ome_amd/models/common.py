@@ -71,8 +71,9 @@ class PagedKVCache:
     def __init__(self, num_layers: int, num_pages: int, num_kv_heads: int, head_dim: int, page_size: int = 16,
                  dtype=torch.bfloat16, device="cuda", v_dim: int | None = None, layers: list[int] | None = None):
         """``v_dim`` = 0: key-only cache (MLA keeps one latent row per token, the values are a
-        slice of it); ``None``: same width as the keys.  ``layers``: the global layer ids held
-        here (a pipeline stage's slice); other entries of ``k`` / ``v`` are None."""
+        slice of it); ``None``: same width as the keys; a {layer: width} map: per layer (0 = that
+        layer keeps key rows only).  ``layers``: the global layer ids held here (a pipeline
+        stage's slice); other entries of ``k`` / ``v`` are None."""
         self.num_layers, self.num_pages, self.page_size = num_layers, num_pages, page_size
         # ``num_kv_heads``: one count, or a {layer: heads} map (DeciLM / Nemotron-NAS: per-layer GQA)
         per = num_kv_heads if isinstance(num_kv_heads, dict) else None
@@ -81,12 +82,14 @@ class PagedKVCache:
         per_d = head_dim if isinstance(head_dim, dict) else None
         head_dim = max(per_d.values()) if per_d else head_dim
         self.head_dim, self.dtype = head_dim, dtype
-        self.v_dim = head_dim if v_dim is None else v_dim
+        per_v = v_dim if isinstance(v_dim, dict) else None
+        self.v_dim = max(per_v.values()) if per_v else (head_dim if v_dim is None else v_dim)
         self.local_layers = list(range(num_layers)) if layers is None else list(layers)
         own = set(self.local_layers)
         hk = (lambda i: per[i]) if per else (lambda i: num_kv_heads)  # noqa: E731
         hd = (lambda i: per_d[i]) if per_d else (lambda i: head_dim)  # noqa: E731
-        vd = (lambda i: per_d[i]) if per_d and v_dim is None else (lambda i: self.v_dim)  # noqa: E731
+        vd = (lambda i: per_v[i]) if per_v else (lambda i: per_d[i]) if per_d and v_dim is None else \
+            (lambda i: self.v_dim)  # noqa: E731
         self.k = [torch.zeros(num_pages, hk(i), page_size, hd(i), dtype=dtype, device=device)
                   if i in own else None for i in range(num_layers)]
         self.v = [torch.zeros(num_pages, hk(i), vd(i), page_size, dtype=dtype, device=device)
@@ -113,7 +116,8 @@ class PagedKVCache:
         esz = torch.tensor([], dtype=dtype).element_size()
         if isinstance(head_dim, dict):   # per-layer widths (values as wide as the keys, or ``v_dim`` for all)
             hk = num_kv_heads if isinstance(num_kv_heads, dict) else {i: num_kv_heads for i in head_dim}
-            return sum(hk[i] * (d + (d if v_dim is None else v_dim)) for i, d in head_dim.items()) * page_size * esz
+            vw = (lambda i, d: v_dim[i]) if isinstance(v_dim, dict) else (lambda i, d: d if v_dim is None else v_dim)  # noqa: E731
+            return sum(hk[i] * (d + vw(i, d)) for i, d in head_dim.items()) * page_size * esz
         v = head_dim if v_dim is None else v_dim
         heads = sum(num_kv_heads.values()) if isinstance(num_kv_heads, dict) else num_layers * num_kv_heads
         return heads * (head_dim + v) * page_size * esz

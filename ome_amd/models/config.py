@@ -169,7 +169,7 @@ def layer_runs(c: dict[str, Any]) -> list[tuple[int, int]]:
 
 
 def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
-    """Layer-list configs (``architecture: Zavilorn`` / ``Metitar`` / ``Milenex``): ``layers`` is a
+    """Layer-list configs (``architecture: Zavilorn`` / ``Metitar`` / ``Milenex`` / ``Nivasun``): ``layers`` is a
     list of blocks, each with its mixer ``type``, the mixer's own sizes and its feed-forward.  The
     standard keys describe the envelope the runtime sizes its workspaces by (widest attention layer,
     fewest kv heads); the model reads the per-layer entries from ``extra``.  ``num_hidden_layers``
@@ -181,11 +181,14 @@ def _layer_list_keys(c: dict[str, Any]) -> dict[str, Any]:
             attn.append(m["left"])
             dims.append(attn_tile_dim(max(m["left"]["dim"], m["left"]["vdim"])))
         elif L.get("type") in ("attention", "attention_2"):
+            if c["architecture"] == "Nivasun" and L["type"] == "attention_2":
+                # two score maps per head run as separate heads: twice the query and key heads
+                m = dict(m, heads=2 * m["heads"], kv_heads=2 * m["kv_heads"])
             attn.append(m)
             dims.append(attn_tile_dim(max(m["dim"], m["vdim"])))
         elif L.get("type") == "latent_attention":   # absorbed form: one shared head of latent + rotary width
             attn.append(m)
-            dims.append(latent_row_width(m["kv_rank"], m["rot_dim"]))
+            dims.append(latent_row_width(m["kv_rank"], m.get("rot_dim", 0)))
     ff = [(L["mlp"].get("ff") or (L["mlp"].get("expert") or {}).get("ff") or 0) for L in c["layers"] if L.get("mlp")]
     D = max(dims or [64])
     out = dict(c)

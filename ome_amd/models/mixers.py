@@ -17,7 +17,11 @@ constructor argument), for decoders that assemble their layers from a per-layer 
 * :class:`InputScaledMoE` -- sigmoid-routed mixture of SwiGLU experts whose router score scales the
   expert's input, plus an optional always-on shared expert;
 * :class:`TokenSideInput` -- a gated per-layer slice of a second token embedding, projected back to
-  the stream.
+  the stream;
+* :class:`KeyValuedAttention` -- grouped-query attention whose values are the unrotated keys, with
+  a per-head temperature, a sliding window and a softmax sink;
+* :class:`DifferentialAttention` -- two softmax maps per head over the same values, the second
+  taken off the first, then a weightless per-head RMS norm.
 
 Each block owns its weights (fused input projection, checkpoint tensors concatenated at load), its
 recurrent state (``alloc_state``) and one ``forward(h, ctx)`` over a varlen batch of rows: prompt
@@ -273,16 +277,21 @@ class LatentAttention(_Block):
       ``ops.latent_prep`` -> ``paged_attention`` (more than 16 heads in groups of 16) -> W_uv.
 
     ``kv_layer`` != ``layer``: this layer has no W_dkv and attends over ``kv_layer``'s cache rows with
-    its own W_uk / W_uv.  Checkpoint tensors ``dq dq.norm uq [dkv dkv.norm] uk uv sink o``."""
+    its own W_uk / W_uv.  ``rot_dim`` = 0: no rotated part at all (no positions).  ``window`` > 0:
+    query i sees keys j with 0 <= i - j < window.  ``sink`` False: an ordinary softmax.  ``gated``:
+    the concatenated heads are multiplied by sigmoid(W_g h) before W_o (W_g rides in the fused
+    input projection).  Checkpoint tensors ``dq dq.norm uq [dkv dkv.norm] uk uv [sink] [g] o``."""
 
     HEAD_GROUP = 16   # query heads per kv head one launch of the generic attention kernels takes
 
     def __init__(self, layer: int, kv_layer: int, width: int, heads: int, dim: int, rot_dim: int, vdim: int,
                  kv_rank: int, q_rank: int, rot_base: float, rot_scaling: dict | None, scale: float, eps: float,
-                 max_positions: int, device, dtype, latent_cache: bool | None = None):
+                 max_positions: int, device, dtype, latent_cache: bool | None = None, window: int = -1,
+                 sink: bool = True, gated: bool = False):
         super().__init__(device, dtype)
-        if rot_dim % 2 or rot_dim <= 0:
-            raise ValueError(f"latent attention: rotary width {rot_dim} must be even and positive")
+        if rot_dim % 2 or rot_dim < 0:
+            raise ValueError(f"latent attention: rotary width {rot_dim} must be even")
+        self.window, self.has_sink, self.gated = int(window) if window and window > 0 else -1, bool(sink), bool(gated)
         self.layer, self.kv_layer, self.width, self.H = layer, kv_layer, width, heads
         self.dim, self.rot, self.vdim, self.R, self.qr = dim, rot_dim, vdim, kv_rank, q_rank
         self.scale, self.eps = float(scale), float(eps)
@@ -299,28 +308,32 @@ class LatentAttention(_Block):
             if dtype != torch.float32 and self.D > 256:
                 raise ValueError(f"latent attention: a {kv_rank} + {rot_dim}-wide row fits neither the latent kernel "
                                  "(latent <= 512, rotary <= 64) nor the 256-wide attention tile")
-        self.cos_sin = yarn_rope_table(rot_base, rot_dim, max_positions, rot_scaling, self.device)
+        self.cos_sin = yarn_rope_table(rot_base, rot_dim, max_positions, rot_scaling, self.device) if rot_dim else \
+            torch.zeros(max_positions, 0, device=self.device)
         self.w_in = self.qn = self.w_uq = self.kvn = self.w_uk = self.w_uv = self.sink = self.w_o = None
 
     def load(self, t: dict) -> None:
         H, R = self.H, self.R
-        self.w_in = self._put(torch.cat([t["dq"], t["dkv"]], 0) if self.own_cache else t["dq"])
+        parts = [t["dq"]] + ([t["dkv"]] if self.own_cache else []) + ([t["g"]] if self.gated else [])
+        self.w_in = self._put(torch.cat(parts, 0))
         self.qn, self.w_uq = self._put(t["dq.norm"]), self._put(t["uq"])
         if self.own_cache:
             self.kvn = self._put(t["dkv.norm"])
         self.w_uk = self._put(t["uk"].view(H, self.dim, R))                       # q_lat = q_nope @ W_uk[h]
         self.w_uv = self._put(t["uv"].view(H, self.vdim, R).transpose(1, 2))      # o = o_lat @ W_uv[h]^T
-        self.sink, self.w_o = self._put(t["sink"], torch.float32), self._put(t["o"])
+        self.sink = self._put(t["sink"], torch.float32) if self.has_sink else None
+        self.w_o = self._put(t["o"])
 
     def init_random(self, gen, std: float) -> None:
         H, R = self.H, self.R
-        self.w_in = self._rand(gen, self.qr + (R + self.rot if self.own_cache else 0), self.width, std=std)
+        self.w_in = self._rand(gen, self.qr + (R + self.rot if self.own_cache else 0) +
+                               (H * self.vdim if self.gated else 0), self.width, std=std)
         self.qn = torch.ones(self.qr, dtype=self.dtype, device=self.device)
         self.w_uq = self._rand(gen, H * (self.dim + self.rot), self.qr, std=std)
         if self.own_cache:
             self.kvn = torch.ones(R, dtype=self.dtype, device=self.device)
         self.w_uk, self.w_uv = self._rand(gen, H, self.dim, R, std=std), self._rand(gen, H, R, self.vdim, std=std)
-        self.sink = torch.zeros(H, dtype=torch.float32, device=self.device)
+        self.sink = torch.zeros(H, dtype=torch.float32, device=self.device) if self.has_sink else None
         self.w_o = self._rand(gen, self.width, H * self.vdim, std=std)
 
     def forward(self, h: torch.Tensor, ctx: MixerCtx) -> torch.Tensor:
@@ -340,16 +353,19 @@ class LatentAttention(_Block):
             ws = _latent_workspace(h)
             for s, e, bt, rows, lens in latent_rows(ctx.meta, T):
                 ops.latent_attn(q_full[s:e], rows3, bt, rows, lens, self.scale, self.DV, ws, out=o_lat[s:e],
-                                sinks=self.sink)
+                                sinks=self.sink, window=self.window)
         else:
             G = self.HEAD_GROUP
             if H <= G:
-                o_lat = paged_attention(q_full, k_cache, v_cache, ctx.meta, self.scale, sinks=self.sink)
+                o_lat = paged_attention(q_full, k_cache, v_cache, ctx.meta, self.scale, self.window, sinks=self.sink)
             else:   # the kernels share one kv head among at most G query heads: run the heads in groups
                 o_lat = torch.cat([paged_attention(q_full[:, g:g + G], k_cache, v_cache, ctx.meta, self.scale,
-                                                   sinks=self.sink[g:g + G]) for g in range(0, H, G)], 1)
+                                                   self.window, sinks=None if self.sink is None else self.sink[g:g + G])
+                                   for g in range(0, H, G)], 1)
         o = torch.empty(T, H * self.vdim, dtype=h.dtype, device=h.device)
         torch.bmm(o_lat[:, :, :R].transpose(0, 1), self.w_uv, out=o.view(T, H, self.vdim).transpose(0, 1))
+        if self.gated:
+            o = ops.head_gate(o.view(T, H, self.vdim), a[:, a.shape[1] - H * self.vdim:], self.vdim, 0)
         return linear(o, self.w_o)
 
 
@@ -688,7 +704,11 @@ class GroupRoutedMoE(_Block):
     by its best choice score; experts of the other groups are excluded outright); the ``top``
     chosen experts' outputs are weighted by their plain scores s (not renormalised).  An optional
     shared expert (own width and ``limit``) runs for every token, times sigmoid(w_sg . h).
-    Checkpoint tensors ``router correction e<j>.gate|up|down [shared.gate|up|down|sg]``.
+    ``act``: the experts' gated activation (2 clamped GLU, 0 plain SiLU GLU: no ``limit``);
+    ``renorm``: the chosen scores are divided by their sum (= a softmax over the chosen logits
+    alone); ``router_bias``: the router has a bias ``router.b`` that is part of the logits;
+    ``correction`` False: no choice-only correction tensor.
+    Checkpoint tensors ``router [router.b] [correction] e<j>.gate|up|down [shared.gate|up|down|sg]``.
 
     The router and the shared gate are one fp32-result GEMM (``[W_r; w_sg]``).  Experts run on the
     grouped MFMA GEMMs (bf16, widths in multiples of 32), otherwise densely: every expert over all
@@ -696,10 +716,15 @@ class GroupRoutedMoE(_Block):
     shape, fp32 models; no host synchronisation either way."""
 
     def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, groups: int, keep: int,
-                 shared_ff: int, shared_limit: float, device, dtype):
+                 shared_ff: int, shared_limit: float, device, dtype, act: int = 2, renorm: bool = False,
+                 router_bias: bool = False, correction: bool = True):
         super().__init__(device, dtype)
         if groups < 1 or experts % groups or not 1 <= keep <= groups or top > keep * (experts // groups):
             raise ValueError(f"moe: {experts} experts in {groups} groups, {keep} kept, top {top}")
+        if experts > 512 or top > 16:
+            raise ValueError(f"moe: {experts} experts / top {top} exceed the router kernel (512 / 16)")
+        self.act, self.renorm, self.has_rb, self.has_corr = int(act), bool(renorm), bool(router_bias), bool(correction)
+        self.router_b = None
         self.width, self.E, self.k, self.ff, self.limit = width, experts, top, ff, float(limit)
         self.groups, self.keep = groups, keep
         self.sff, self.slimit = int(shared_ff or 0), float(shared_limit or 0.0)
@@ -708,7 +733,8 @@ class GroupRoutedMoE(_Block):
     def load(self, t: dict) -> None:
         self.w_router = self._put(torch.cat([t["router"], t["shared.sg"].reshape(1, -1)], 0) if self.sff
                                   else t["router"])
-        self.correction = self._put(t["correction"], torch.float32)
+        self.correction = self._put(t["correction"], torch.float32) if self.has_corr else None
+        self.router_b = self._put(t["router.b"], torch.float32) if self.has_rb else None
         self.w13 = self._put(torch.stack([torch.cat([t[f"e{e}.gate"], t[f"e{e}.up"]], 0) for e in range(self.E)]))
         self.w2 = self._put(torch.stack([t[f"e{e}.down"] for e in range(self.E)]))
         if self.sff:
@@ -716,7 +742,8 @@ class GroupRoutedMoE(_Block):
 
     def init_random(self, gen, std: float) -> None:
         self.w_router = self._rand(gen, self.E + (1 if self.sff else 0), self.width, std=std)
-        self.correction = torch.zeros(self.E, dtype=torch.float32, device=self.device)
+        self.correction = torch.zeros(self.E, dtype=torch.float32, device=self.device) if self.has_corr else None
+        self.router_b = torch.zeros(self.E, dtype=torch.float32, device=self.device) if self.has_rb else None
         self.w13, self.w2 = self._rand(gen, self.E, 2 * self.ff, self.width, std=std), self._rand(
             gen, self.E, self.width, self.ff, std=std)
         if self.sff:
@@ -729,17 +756,134 @@ class GroupRoutedMoE(_Block):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         T, W = h.shape
         logits = ops.lm_head_f32(h, self.w_router)                        # fp32 [T, E (+ shared gate)]
-        tw, tid = ops.moe_route(logits[:, :self.E], self.k, False, "softmax", bias=self.correction,
-                                n_group=self.groups, topk_group=self.keep, group_mode=3 if self.groups > 1 else 0)
+        tw, tid = ops.moe_route(logits[:, :self.E], self.k, self.renorm, "softmax", bias=self.correction,
+                                n_group=self.groups, topk_group=self.keep, group_mode=3 if self.groups > 1 else 0,
+                                logit_bias=self.router_b)
         sh = None
         if self.sff:
-            a = ops.act_and_mul(linear(h, self.w_sgu).contiguous(), 2, limit=self.slimit, row_gate=logits[:, self.E])
+            a = ops.act_and_mul(linear(h, self.w_sgu).contiguous(), self.act, limit=self.slimit,
+                                row_gate=logits[:, self.E])
             sh = linear(a, self.w_sd)
         if self.grouped_ok(h):
-            return ops.fused_moe(h, tw, tid, self.w13, self.w2, act=2, limit=self.limit,
+            return ops.fused_moe(h, tw, tid, self.w13, self.w2, act=self.act, limit=self.limit,
                                  add=sh.contiguous() if sh is not None else None)
         wd = torch.zeros(T, self.E, dtype=torch.float32, device=h.device).scatter_(1, tid.long(), tw)
         gu = torch.matmul(h, self.w13.transpose(1, 2))                    # [E, T, 2 ff]
-        hh = ops.act_and_mul(gu.view(self.E * T, 2 * self.ff), 2, limit=self.limit).view(self.E, T, self.ff)
+        hh = ops.act_and_mul(gu.view(self.E * T, 2 * self.ff), self.act, limit=self.limit).view(self.E, T, self.ff)
         y = (torch.bmm(hh, self.w2.transpose(1, 2)).float() * wd.t()[:, :, None]).sum(0)
         return (y if sh is None else y + sh.float()).to(h.dtype)
+
+
+class KeyValuedAttention(_Block):
+    """Grouped-query attention without a value projection: q = W_q h, k = W_k h, and the values
+    are the keys as projected (v = k BEFORE the rotation).  q and k are rotated on the first
+    ``rot_dims`` dims of every head (half-split pairs i / i + rot_dims/2 by default, or
+    ``interleaved`` neighbours); score = q.k * ``scale`` * temp_h (a learned per-head temperature);
+    query i sees keys j with 0 <= i - j < ``window``; softmax whose denominator also holds
+    exp(``sink``_h) (not scaled, not multiplied by the temperature); W_o on the concatenated heads.
+    Checkpoint tensors ``q k temp sink o``.  The temperature is folded into the rotated query in
+    fp32 before its one rounding (``ops.wide_norm_rope_cache(q_scale=)``), the key projection is
+    written into the paged cache twice: rotated as the key row, unrotated as the value column."""
+
+    def __init__(self, layer: int, width: int, heads: int, kv_heads: int, dim: int, window: int, rot_base: float,
+                 rot_dims: int, scale: float, max_positions: int, device, dtype, interleaved: bool = False):
+        super().__init__(device, dtype)
+        if heads % kv_heads or heads // kv_heads > 16:
+            raise ValueError(f"attention: {heads} query heads over {kv_heads} kv heads (groups of <= 16 supported)")
+        self.layer, self.width, self.Hq, self.Hkv, self.dim = layer, width, heads, kv_heads, dim
+        self.window = int(window) if window and window > 0 else -1
+        self.rot_dims, self.scale, self.interleaved = int(rot_dims), float(scale), bool(interleaved)
+        self.D = attn_tile_dim(dim)
+        self.cos_sin = plain_rope_table(rot_base, self.rot_dims, max_positions, self.device) if rot_dims else \
+            torch.zeros(max_positions, 0, device=self.device)
+        self.nq, self.nk = heads * dim, kv_heads * dim
+        self.w_in = self.temp = self.sink = self.w_o = None
+
+    def load(self, t: dict) -> None:
+        self.w_in = self._put(torch.cat([t["q"], t["k"]], 0))
+        self.temp, self.sink = self._put(t["temp"], torch.float32), self._put(t["sink"], torch.float32)
+        self.w_o = self._put(t["o"])
+        if tuple(self.w_in.shape) != (self.nq + self.nk, self.width) or self.temp.numel() != self.Hq:
+            raise ValueError(f"attention: q / k {tuple(self.w_in.shape)} or temp {tuple(self.temp.shape)} do not fit "
+                             f"{self.Hq} + {self.Hkv} heads of {self.dim}")
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_in = self._rand(gen, self.nq + self.nk, self.width, std=std)
+        self.temp = torch.linspace(0.75, 1.25, self.Hq, dtype=torch.float32, device=self.device)
+        self.sink = torch.zeros(self.Hq, dtype=torch.float32, device=self.device)
+        self.w_o = self._rand(gen, self.width, self.nq, std=std)
+
+    def forward(self, h: torch.Tensor, ctx: MixerCtx) -> torch.Tensor:
+        T, nq = h.shape[0], self.nq
+        p = linear(h, self.w_in)                                   # [T, q | k]
+        q = torch.empty(T, self.Hq, self.D, dtype=h.dtype, device=h.device)
+        k_cache, v_cache = ctx.kv.layer(self.layer)
+        ops.wide_norm_rope_cache(p[:, :nq], p[:, nq:], p[:, nq:], ctx.meta.positions, self.cos_sin, self.rot_dims,
+                                 self.interleaved, None, None, 0.0, q, k_cache, v_cache, ctx.meta.slots, self.Hq,
+                                 self.Hkv, self.dim, self.dim, q_scale=self.temp)
+        a = paged_attention(q, k_cache, v_cache, ctx.meta, self.scale, self.window, 0, self.sink)
+        if self.D != self.dim:
+            a = a[:, :, :self.dim].reshape(T, nq)
+        return linear(a.view(T, nq), self.w_o)
+
+
+class DifferentialAttention(_Block):
+    """Differential attention.  q = W_q h has ``heads`` x 2 x ``dim`` rows and k = W_k h ``kv_heads``
+    x 2 x ``dim``, head by head as [map 1, map 2]; v = W_v h has ``kv_heads`` x ``vdim``.  Every map is
+    rotated on its first ``rot_dims`` dims (interleaved pairs by default) and is a windowed softmax
+    attention of its own (score = q.k * ``scale``, 0 <= i - j < ``window``) over the head's values;
+    with lam = exp(lq1 . lk1) - exp(lq2 . lk2) + ``diff`` (one number per layer): o = a1 - lam a2,
+    o / sqrt(mean(o^2) + eps) over ``vdim`` (no weight), times (1 - ``diff``); W_o.  Checkpoint
+    tensors ``q k v lq1 lk1 lq2 lk2 o``.
+
+    The maps run as separate heads of the framework's paged attention kernels: 2 x ``heads`` query
+    heads over 2 x ``kv_heads`` key heads.  The rows of W_q are reordered at load to [kv group][map]
+    [head of the group], so that query head (g, m, r) reads key head 2 g + m, which is where k's
+    layout already has it; the cache holds the group's values under both key heads (``v_rep`` =
+    2).  ``ops.diff_head_norm`` then combines the two outputs of a head, norms and rounds once."""
+
+    def __init__(self, layer: int, width: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int,
+                 rot_base: float, rot_dims: int, scale: float, diff: float, eps: float, max_positions: int, device,
+                 dtype, interleaved: bool = True):
+        super().__init__(device, dtype)
+        if heads % kv_heads or heads // kv_heads > 16:
+            raise ValueError(f"attention: {heads} query heads over {kv_heads} kv heads (groups of <= 16 supported)")
+        self.layer, self.width, self.H, self.G, self.dim, self.vdim = layer, width, heads, kv_heads, dim, vdim
+        self.Hq, self.Hkv, self.group = 2 * heads, 2 * kv_heads, heads // kv_heads
+        self.window = int(window) if window and window > 0 else -1
+        self.rot_dims, self.scale, self.diff, self.eps = int(rot_dims), float(scale), float(diff), float(eps)
+        self.interleaved = bool(interleaved)
+        self.D = attn_tile_dim(max(dim, vdim))
+        self.cos_sin = plain_rope_table(rot_base, self.rot_dims, max_positions, self.device) if rot_dims else \
+            torch.zeros(max_positions, 0, device=self.device)
+        self.nq, self.nk, self.nv = 2 * heads * dim, 2 * kv_heads * dim, kv_heads * vdim
+        self.lam = float(diff)
+        self.w_in = self.w_o = None
+
+    def load(self, t: dict) -> None:
+        G, R, d = self.G, self.group, self.dim
+        wq = t["q"]
+        if tuple(wq.shape) != (self.nq, self.width):
+            raise ValueError(f"attention_2: q {tuple(wq.shape)} != [{self.nq}, {self.width}]")
+        wq = wq.view(G, R, 2, d, self.width).permute(0, 2, 1, 3, 4).reshape(self.nq, self.width)
+        self.w_in = self._put(torch.cat([wq, t["k"], t["v"]], 0))
+        f = lambda n: t[n].double()   # noqa: E731
+        self.lam = math.exp(float((f("lq1") * f("lk1")).sum())) - math.exp(float((f("lq2") * f("lk2")).sum())) + self.diff
+        self.w_o = self._put(t["o"])
+
+    def init_random(self, gen, std: float) -> None:
+        self.w_in = self._rand(gen, self.nq + self.nk + self.nv, self.width, std=std)
+        self.lam = self.diff
+        self.w_o = self._rand(gen, self.width, self.H * self.vdim, std=std)
+
+    def forward(self, h: torch.Tensor, ctx: MixerCtx) -> torch.Tensor:
+        T, nq, nk = h.shape[0], self.nq, self.nk
+        p = linear(h, self.w_in)                                   # [T, q (group, map, head) | k | v]
+        q = torch.empty(T, self.Hq, self.D, dtype=h.dtype, device=h.device)
+        k_cache, v_cache = ctx.kv.layer(self.layer)
+        ops.wide_norm_rope_cache(p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:], ctx.meta.positions, self.cos_sin,
+                                 self.rot_dims, self.interleaved, None, None, 0.0, q, k_cache, v_cache, ctx.meta.slots,
+                                 self.Hq, self.Hkv, self.dim, self.vdim, v_rep=2)
+        a = paged_attention(q, k_cache, v_cache, ctx.meta, self.scale, self.window)
+        o = ops.diff_head_norm(a, self.lam, self.eps, 1.0 - self.diff, self.group, self.vdim)
+        return linear(o, self.w_o)

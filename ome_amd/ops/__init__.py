@@ -303,6 +303,43 @@ def embedding_f32(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) ->
     return out
 
 
+def pair_embedding_f32(ids: torch.Tensor, table: torch.Tensor, scale: float, pair: torch.Tensor, buckets: int,
+                       mul_prev: int, mul_cur: int, state: torch.Tensor, seqs: tuple) -> torch.Tensor:
+    """fp32 [T, H] rows ``table[id] * scale + pair[r]`` with a hashed token-pair row: ``r = (previous
+    id * mul_prev + id * mul_cur) mod buckets``, or row ``buckets`` (the table's last) for a
+    sequence's first token.  The id before a chunk's first row is ``state[slot]`` (int32 [slots]);
+    the chunk's last id replaces it (``seqs`` = (cu, slot, reset), ``reset``: the sequence starts)."""
+    cu, slot, reset = seqs
+    assert pair.shape[0] == buckets + 1 and pair.shape[1] == table.shape[1] and state.dtype == torch.int32
+    if not _gpu(ids):
+        return ref.pair_embedding_f32(ids, table, scale, pair, buckets, mul_prev, mul_cur, state, cu, slot, reset)
+    T, H = ids.shape[0], table.shape[1]
+    assert table.is_contiguous() and pair.is_contiguous() and state.is_contiguous()
+    out = torch.empty(T, H, dtype=torch.float32, device=table.device)
+    call("ome_pair_embedding_f32", _i32(ids).data_ptr(), table.data_ptr(), pair.data_ptr(), out.data_ptr(),
+         state.data_ptr(), T, H, table.shape[0], float(scale), int(buckets), int(mul_prev), int(mul_cur),
+         _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], _f32(table, pair),
+         stream_ptr())
+    return out
+
+
+def diff_head_norm(a: torch.Tensor, lam: float, eps: float, out_scale: float, group: int, vdim: int) -> torch.Tensor:
+    """Combine of a two-map (differential) attention: ``a`` [T, 2 * H, D] holds, for every kv group g
+    (``group`` query heads each), the first map's outputs of the group's heads and then the second
+    map's: head h = g * group + r has a1 = a[:, 2 g * group + r], a2 = a[:, (2 g + 1) * group + r].
+    Returns ``(a1 - lam * a2) / sqrt(mean((a1 - lam * a2)^2) + eps) * out_scale`` over the first
+    ``vdim`` columns as a contiguous [T, H * vdim] (fp32 inside, one rounding)."""
+    T, H2, D = a.shape
+    assert H2 % (2 * group) == 0 and vdim <= D
+    if not _gpu(a):
+        return ref.diff_head_norm(a, lam, eps, out_scale, group, vdim)
+    assert a.is_contiguous()
+    out = torch.empty(T, (H2 // 2) * vdim, dtype=a.dtype, device=a.device)
+    call("ome_diff_head_norm", a.data_ptr(), out.data_ptr(), T, H2 // 2, int(group), D, int(vdim), float(lam),
+         float(eps), float(out_scale), _f32(a), stream_ptr())
+    return out
+
+
 def residual_rmsnorm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor | None = None,
                      s1: float = 1.0, x2: torch.Tensor | None = None, s2: float = 1.0,
                      out_dtype=None) -> torch.Tensor:
@@ -327,7 +364,8 @@ def residual_rmsnorm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.T
 
 
 def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim: int, interleaved: bool, qn_w, kn_w, eps: float,
-                         q_out, k_cache, v_cache, slots, Hq: int, Hkv: int, dim: int, vdim: int) -> None:
+                         q_out, k_cache, v_cache, slots, Hq: int, Hkv: int, dim: int, vdim: int,
+                         q_scale: torch.Tensor | None = None, v_rep: int = 1) -> None:
     """q [T, Hq*dim], k [T, Hkv*dim], v [T, Hkv*vdim] (row-strided views of a fused projection) ->
     projection-wide RMSNorm of q and of k (ONE root mean square over all heads' channels of a row,
     weights ``qn_w`` / ``kn_w`` of the projection's width, None = no norm), rotary embedding on the
@@ -335,12 +373,16 @@ def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim: int, interleaved:
     i + rot_dim/2; angles from the ``cos_sin`` table row of the token's position), q into
     ``q_out`` [T, Hq, D], k / v into the paged cache at ``slots``.  ``dim`` / ``vdim`` <= D (the
     cache's head width): the tail of every head is written as zeros, which adds nothing to a score
-    and leaves the padded output columns zero."""
+    and leaves the padded output columns zero.  ``q_scale``: fp32 [Hq], every query head is
+    multiplied by its factor (a per-head temperature; fp32, before the one rounding).  ``v_rep``
+    > 1: v holds Hkv / v_rep value heads and cache head h stores value head h // v_rep (several
+    key heads that attend over the same values)."""
     P, D = k_cache.shape[2], k_cache.shape[3]
     assert dim <= D and vdim <= D and rot_dim <= dim and rot_dim % 2 == 0
+    assert v_rep >= 1 and Hkv % v_rep == 0 and v.shape[1] >= (Hkv // v_rep) * vdim
     if not _gpu(q):
         return ref.wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim, interleaved, qn_w, kn_w, eps, q_out,
-                                        k_cache, v_cache, slots, Hq, Hkv, dim, vdim, P)
+                                        k_cache, v_cache, slots, Hq, Hkv, dim, vdim, P, q_scale, v_rep)
     f32 = _f32(q, k, v, qn_w, kn_w, q_out, k_cache, v_cache)
     assert q_out.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()
     assert q.stride(1) == k.stride(1) == v.stride(1) == 1 and cos_sin.dtype == torch.float32
@@ -348,7 +390,7 @@ def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim: int, interleaved:
     call("ome_wide_norm_rope_cache", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
          _i32(positions).data_ptr(), cos_sin.data_ptr(), int(rot_dim), int(bool(interleaved)), ptr(qn_w), ptr(kn_w),
          float(eps), q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _i32(slots).data_ptr(), q.shape[0],
-         Hq, Hkv, dim, vdim, D, P, f32, stream_ptr())
+         Hq, Hkv, dim, vdim, D, P, f32, _sinks(q_scale), int(v_rep), stream_ptr())
 
 
 def head_gate(o: torch.Tensor, g: torch.Tensor, vdim: int, kind: int = 0) -> torch.Tensor:
@@ -592,13 +634,15 @@ def fp8_linear(x: torch.Tensor, qw: torch.Tensor, sw: torch.Tensor, block: int =
 
 def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, scoring: str = "softmax",
               out_w: torch.Tensor | None = None, out_ids: torch.Tensor | None = None, bias: torch.Tensor | None = None,
-              n_group: int = 1, topk_group: int = 1, group_mode: int = 0):
-    """Router: logits [T, E] -> (weights f32 [T, k], expert ids int32 [T, k]).  ``group_mode`` 1/2 =
+              n_group: int = 1, topk_group: int = 1, group_mode: int = 0, logit_bias: torch.Tensor | None = None):
+    """Router: logits [T, E] -> (weights f32 [T, k], expert ids int32 [T, k]).  ``logit_bias``: fp32
+    [E] added to the logits themselves (it counts in the scores and weights, unlike ``bias``,
+    which only steers the choice).  ``group_mode`` 1/2 =
     DeepSeek-V2 group_limited_greedy / DeepSeek-V3 noaux_tc (with ``bias``); 3 = a group scores by
     its best biased expert and the experts of unchosen groups are excluded outright (minus
     infinity where modes 1 / 2 set them to 0, which a negative biased score would lose against)."""
     if not _gpu(logits):
-        w, ids = ref.moe_route(logits, k, renorm, scoring, bias, n_group, topk_group, group_mode)
+        w, ids = ref.moe_route(logits, k, renorm, scoring, bias, n_group, topk_group, group_mode, logit_bias)
         if out_w is not None:
             out_w.copy_(w)
             out_ids.copy_(ids)
@@ -607,11 +651,11 @@ def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, scoring: str = 
     T, E = logits.shape
     out_w = torch.empty(T, k, dtype=torch.float32, device=logits.device) if out_w is None else out_w
     out_ids = torch.empty(T, k, dtype=torch.int32, device=logits.device) if out_ids is None else out_ids
-    if bias is not None:
-        assert bias.dtype == torch.float32 and bias.is_contiguous()
+    for b in (bias, logit_bias):
+        assert b is None or (b.dtype == torch.float32 and b.is_contiguous() and b.numel() == E)
     call("ome_moe_route", logits.data_ptr(), int(logits.dtype == torch.bfloat16), logits.stride(0), T, E, k,
          int(renorm), 0 if scoring == "softmax" else 1, ptr(bias), n_group, topk_group, group_mode,
-         out_w.data_ptr(), out_ids.data_ptr(), stream_ptr())
+         out_w.data_ptr(), out_ids.data_ptr(), ptr(logit_bias), stream_ptr())
     return out_w, out_ids
 
 
@@ -1732,18 +1776,19 @@ def post_norm_add(res: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.
 
 
 def conv_mix(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor, cu, slot, reset, out_dtype) -> torch.Tensor:
-    """``x + causal_conv(x)`` per channel over a varlen batch of an fp32 stream: x [T, C] fp32, taps
-    w [C, K] (tap K-1 on the current row, no bias, no activation), ``state`` [slots, C, K-1] fp32 =
-    the last K-1 input rows of each sequence, continued / updated (``reset[s]``: start from zeros)."""
+    """``x + causal_conv(x)`` per channel over a varlen batch: x [T, C] fp32 (a residual stream) or
+    the taps' dtype (a normed row already rounded for the GEMMs), taps w [C, K] (tap K-1 on the
+    current row, no bias, no activation), ``state`` [slots, C, K-1] fp32 = the last K-1 input rows
+    of each sequence, continued / updated (``reset[s]``: start from zeros).  Sums are fp32."""
     T, C = x.shape
     out = torch.empty(T, C, dtype=out_dtype, device=x.device)
     if not _gpu(x):
         return ref.conv_mix(x, w, state, cu, slot, reset, out)
-    assert x.dtype == torch.float32 and state.dtype == torch.float32 and x.stride(1) == 1
+    assert x.dtype in (torch.float32, w.dtype) and state.dtype == torch.float32 and x.stride(1) == 1
     assert w.is_contiguous() and state.is_contiguous() and state.shape[1:] == (C, w.shape[1] - 1)
     call("ome_conv_mix", x.data_ptr(), x.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0), state.data_ptr(),
          _i32(cu).data_ptr(), _i32(slot).data_ptr(), _i32(reset).data_ptr(), slot.shape[0], T, C, w.shape[1],
-         _f32(w, out), stream_ptr())
+         _f32(w, out), int(x.dtype == torch.float32), stream_ptr())
     return out
 
 
@@ -1796,14 +1841,15 @@ def latent_shape(lat: int, rope: int) -> tuple[int, int] | None:
 
 
 def latent_attn(q, cache, block_tables, tok_row, kv_lens, scale: float, dv: int, ws: MLAWorkspace | None = None,
-                out: torch.Tensor | None = None, sinks: torch.Tensor | None = None) -> torch.Tensor:
+                out: torch.Tensor | None = None, sinks: torch.Tensor | None = None, window: int = -1) -> torch.Tensor:
     """Absorbed latent attention over a paged cache of key rows that carry their own values: q [T,
     H, DK], cache [pages, 16, DK] -> out [T, H, dv] (values = the first ``dv`` columns of a row);
     (DK, dv) one of :data:`LATENT_SHAPES`.  Token t sees keys [0, kv_lens[t]) of block-table row
     tok_row[t] (prompt chunks, decode rows and mixed batches alike).  ``sinks``: fp32 [H] logits
-    that join each head's softmax denominator (no key, no value, unscaled)."""
+    that join each head's softmax denominator (no key, no value, unscaled).  ``window`` > 0: only
+    the last ``window`` of those keys, [kv_lens[t] - window, kv_lens[t])."""
     if not _gpu(q):
-        r = ref.mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv, sinks)
+        r = ref.mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv, sinks, window)
         if out is not None:
             out.copy_(r)
             return out
@@ -1816,14 +1862,14 @@ def latent_attn(q, cache, block_tables, tok_row, kv_lens, scale: float, dv: int,
         out = torch.empty(T, H, dv, dtype=q.dtype, device=q.device)
     assert out.stride(2) == 1 and out.stride(1) == dv
     parts = MLAWorkspace.parts(T, H, DK)
-    if sinks is not None and DK == 576:   # (sinks run the 16-head kernel: partition as it does)
+    if (sinks is not None or window > 0) and DK == 576:   # (these run the 16-head kernel: partition as it does)
         parts = MLAWorkspace.parts(T, H, 0)
     if parts > 1 and ws is None:
         ws = MLAWorkspace(q.device)
     call("ome_latent_attn", q.data_ptr(), q.stride(0), cache.data_ptr(), _i32(block_tables).data_ptr(),
          block_tables.stride(0), _i32(tok_row).data_ptr(), _i32(kv_lens).data_ptr(), T, H, DK, dv, float(scale),
          parts, out.data_ptr(), out.stride(0), ws.ws_o.data_ptr() if parts > 1 else None,
-         ws.ws_ml.data_ptr() if parts > 1 else None, _sinks(sinks), stream_ptr())
+         ws.ws_ml.data_ptr() if parts > 1 else None, _sinks(sinks), int(window), stream_ptr())
     return out
 
 
@@ -1910,9 +1956,9 @@ def row_norm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, eps: floa
 def shift_norm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor | None = None, s1: float = 1.0,
                x2: torch.Tensor | None = None, s2: float = 1.0, w_offset: float = 0.0,
                shift: torch.Tensor | None = None, state: torch.Tensor | None = None, seqs: tuple | None = None,
-               out_dtype=None) -> tuple[torch.Tensor, torch.Tensor]:
+               out_dtype=None, bias: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
     """Pre-norm step of an fp32 residual stream, optionally with a token shift.  ``v = res + s1 x1 +
-    s2 x2`` (either addend may be None), ``n = v / sqrt(mean(v^2) + eps) * (w_offset + w)`` (``w_offset``
+    s2 x2 + bias`` (either addend may be None; ``bias`` [H]: one row added to every row, None: none), ``n = v / sqrt(mean(v^2) + eps) * (w_offset + w)`` (``w_offset``
     = 1 for weights stored as the offset from one), and with ``shift`` [H]: ``out[t] = n[t] +
     (n[t-1] - n[t]) * shift`` where the row before a sequence's first row of the step is ``state[slot]``
     ([slots, H] fp32; zeros when the sequence starts) and the sequence's last n replaces it
@@ -1920,7 +1966,7 @@ def shift_norm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor 
     at the end.  Returns (v, out): with a shift v is a NEW tensor (a row's workgroup also reads the
     inputs of the row before it), without one ``res`` is updated in place and returned."""
     if not _gpu(res):
-        v, out = ref.shift_norm(res, w, eps, x1, s1, x2, s2, w_offset, shift, state, seqs, out_dtype)
+        v, out = ref.shift_norm(res, w, eps, x1, s1, x2, s2, w_offset, shift, state, seqs, out_dtype, bias)
         if shift is None:
             res.copy_(v)
             return res, out
@@ -1931,7 +1977,8 @@ def shift_norm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor 
         x1, s1, x2, s2 = x2, s2, None, 1.0
     for a in (x1, x2):
         assert a is None or (a.shape == res.shape and a.stride(1) == 1)
-    f32 = _f32(w, x1, x2, shift)
+    f32 = _f32(w, x1, x2, shift, bias)
+    assert bias is None or (bias.shape == (H,) and bias.is_contiguous())
     out = torch.empty(T, H, dtype=w.dtype, device=res.device)
     if shift is not None:
         cu, slot, reset = seqs
@@ -1944,7 +1991,8 @@ def shift_norm(res: torch.Tensor, w: torch.Tensor, eps: float, x1: torch.Tensor 
         new, sargs = res, (None, None, None, None, None, 0)
     call("ome_shift_norm", res.data_ptr(), new.data_ptr(), res.stride(0), ptr(x1),
          x1.stride(0) if x1 is not None else 0, float(s1), ptr(x2), x2.stride(0) if x2 is not None else 0, float(s2),
-         w.data_ptr(), float(w_offset), *sargs, out.data_ptr(), out.stride(0), T, H, float(eps), f32, stream_ptr())
+         w.data_ptr(), float(w_offset), *sargs, out.data_ptr(), out.stride(0), T, H, float(eps), f32, ptr(bias),
+         stream_ptr())
     return new, out
 
 

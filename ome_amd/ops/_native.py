@@ -41,7 +41,9 @@ _SIGNATURES = {
         "ome_embedding_f32": [vp, vp, vp, i32, i32, i32, f32, i32, vp],
         "ome_residual_rmsnorm": [vp, i64, vp, i64, f32, vp, i64, f32, vp, vp, i64, i32, i32, f32, i32, vp],
         "ome_wide_norm_rope_cache": [vp, i64, vp, i64, vp, i64, vp, vp, i32, i32, vp, vp, f32, vp, vp, vp, vp, i32,
-                                     i32, i32, i32, i32, i32, i32, i32, vp],
+                                     i32, i32, i32, i32, i32, i32, i32, vp, i32, vp],
+        "ome_pair_embedding_f32": [vp, vp, vp, vp, vp, i32, i32, i32, f32, i32, i64, i64, vp, vp, vp, i32, i32, vp],
+        "ome_diff_head_norm": [vp, vp, i32, i32, i32, i32, i32, f32, f32, f32, i32, vp],
         "ome_head_gate": [vp, vp, i64, vp, i32, i32, i32, i32, i32, i32, vp],
         "ome_paged_attention_f32": [vp, i64, vp, vp, vp, i32, vp, vp, vp, i64, i32, i32, i32, i32, i32, f32, i32,
                                     i32, vp, vp],
@@ -50,16 +52,16 @@ _SIGNATURES = {
         "ome_polynorm": [vp, i64, vp, vp, i64, i32, i32, f32, i32, vp],
         "ome_gelu_gather_mul": [vp, i64, vp, vp, i64, i32, i32, vp, i32, i32, i32, vp],
         "ome_scale_rows": [vp, i64, vp, i32, vp, i32, i32, i32, vp],
-        "ome_conv_mix": [vp, i64, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
+        "ome_conv_mix": [vp, i64, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "ome_latent_prep": [vp, i64, i32, i32, i32, vp, f32, vp, vp, vp, vp, vp, i32, i32, i32, vp, i64, i64, i32, i32,
                             vp, i64, i64, i32, i32, vp],
-        "ome_latent_attn": [vp, i64, vp, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32, vp, i64, vp, vp, vp, vp],
+        "ome_latent_attn": [vp, i64, vp, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32, vp, i64, vp, vp, vp, i32, vp],
         "ome_hgrn2_scan": [vp, vp, vp, i64, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, f32, i32, vp],
         "ome_act": [vp, i64, i32, vp],
         "ome_act_any": [vp, i64, i32, i32, vp],
         "ome_act_and_mul_rowgate": [vp, vp, i64, i32, i32, f32, vp, i64, vp],
         "ome_shift_norm": [vp, vp, i64, vp, i64, f32, vp, i64, f32, vp, f32, vp, vp, vp, vp, vp, i32, vp, i64, i32,
-                           i32, f32, i32, vp],
+                           i32, f32, i32, vp, vp],
         "ome_conv_rope_cache": [vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, vp, vp, vp, vp, i32, vp, vp, i32, i32, i32,
                                 f32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "ome_conv_rope_cache_vec": [vp, i64, vp, i64, vp, i64, vp, vp, vp, i32, vp, vp, vp, vp, i32, vp, vp, vp, vp, i32,
@@ -82,7 +84,7 @@ _SIGNATURES = {
         "ome_fill_pending": [vp, vp, vp, i32, vp],
         "ome_apply_penalties": [vp, i32, i64, i32, i32, vp, i64, vp, vp, vp, vp, vp],
         "ome_update_counts": [vp, i64, vp, vp, vp, vp, vp, i32, vp],
-        "ome_moe_route": [vp, i32, i64, i32, i32, i32, i32, i32, vp, i32, i32, i32, vp, vp, vp],
+        "ome_moe_route": [vp, i32, i64, i32, i32, i32, i32, i32, vp, i32, i32, i32, vp, vp, vp, vp],
         "ome_mla_attn": [vp, i64, vp, vp, i32, vp, vp, i32, i32, i32, i32, f32, i32, vp, i64, vp, vp, vp],
         "ome_moe_align": [vp, i32, i32, vp, vp, vp, vp],
         "ome_moe_gemm": [vp, i64, vp, i32, vp, vp, i32, i32, i32, i32, vp, i64, vp, i32, vp],

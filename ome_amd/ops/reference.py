@@ -256,6 +256,32 @@ def embedding_f32(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch
     return table[ids.long()].float() * float(scale)
 
 
+def pair_embedding_f32(ids, table, scale, pair, buckets, mul_prev, mul_cur, state, cu, slot, reset):
+    """``table[id] * scale + pair[(previous id * mul_prev + id * mul_cur) % buckets]`` (row
+    ``buckets`` for a sequence's first token); the id before a chunk is ``state[slot]``."""
+    idl = ids.long()
+    x = table[idl].float() * float(scale)
+    rows = torch.empty_like(idl)
+    for s in range(len(slot)):
+        r0, r1 = int(cu[s]), int(cu[s + 1])
+        if r1 <= r0:
+            continue
+        prev = torch.cat([state[int(slot[s])].view(1).long(), idl[r0:r1 - 1]])
+        rows[r0:r1] = (prev * int(mul_prev) + idl[r0:r1] * int(mul_cur)) % int(buckets)
+        if int(reset[s]):
+            rows[r0] = buckets
+        state[int(slot[s])] = ids[r1 - 1]
+    return x + pair[rows].float()
+
+
+def diff_head_norm(a, lam, eps, out_scale, group, vdim):
+    T, H2, D = a.shape
+    v = a.float().view(T, H2 // (2 * group), 2, group, D)[..., :vdim]
+    o = v[:, :, 0] - float(lam) * v[:, :, 1]
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * float(out_scale)
+    return o.reshape(T, (H2 // 2) * vdim).to(a.dtype)
+
+
 def residual_rmsnorm(res, w, eps, x1=None, s1=1.0, x2=None, s2=1.0, out_dtype=None):
     """fp32 residual stream: ``res += s1 * x1 + s2 * x2`` in place (either addend may be None),
     then returns ``rmsnorm(res) * w`` in ``out_dtype``; everything in fp32 before the final cast."""
@@ -266,7 +292,7 @@ def residual_rmsnorm(res, w, eps, x1=None, s1=1.0, x2=None, s2=1.0, out_dtype=No
 
 
 def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim, interleaved, qn_w, kn_w, eps, q_out, k_cache, v_cache,
-                         slots, Hq, Hkv, dim, vdim, P) -> None:
+                         slots, Hq, Hkv, dim, vdim, P, q_scale=None, v_rep=1) -> None:
     """Projection-wide q / k RMSNorm (one root mean square over ALL heads' channels of a row),
     partial rotary on the first ``rot_dim`` dims of every head (``interleaved``: dim 2i pairs
     with 2i+1; otherwise i with i + rot_dim/2), then q -> ``q_out`` [T, Hq, D] and k / v into the
@@ -297,6 +323,8 @@ def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim, interleaved, qn_w
         return x
 
     qf, kf = prep(q, qn_w, Hq), prep(k, kn_w, Hkv)
+    if q_scale is not None:
+        qf = qf * q_scale.float().view(1, Hq, 1)
     q_out.zero_()
     q_out[:, :, :dim] = qf.to(q_out.dtype)
     ok = slots >= 0
@@ -305,7 +333,8 @@ def wide_norm_rope_cache(q, k, v, positions, cos_sin, rot_dim, interleaved, qn_w
     kp = torch.zeros(int(ok.sum()), Hkv, D, dtype=k_cache.dtype, device=k_cache.device)
     kp[:, :, :dim] = kf[ok].to(k_cache.dtype)
     vp = torch.zeros(int(ok.sum()), Hkv, D, dtype=v_cache.dtype, device=v_cache.device)
-    vp[:, :, :vdim] = v.reshape(T, Hkv, vdim)[ok].to(v_cache.dtype)
+    vp[:, :, :vdim] = v[:, :(Hkv // v_rep) * vdim].reshape(T, Hkv // v_rep, vdim).repeat_interleave(v_rep, 1)[ok].to(
+        v_cache.dtype)
     k_cache[page, :, off, :] = kp
     v_cache[page, :, :, off] = vp
 
@@ -519,11 +548,11 @@ def pool(hidden, cu_lens, mode: int = 0, normalize: bool = True) -> torch.Tensor
 
 # ------------------------------------------------------------------ MoE
 def moe_route(logits, k: int, renorm: bool, scoring: str = "softmax", bias=None, n_group: int = 1,
-              topk_group: int = 1, group_mode: int = 0):
+              topk_group: int = 1, group_mode: int = 0, logit_bias=None):
     """HF semantics (Mixtral/Qwen softmax top-k; DeepSeek-V2 group_limited_greedy = mode 1,
     DeepSeek-V3 noaux_tc = mode 2 with e_score_correction_bias; mode 3 = the group's best
     biased score, experts of the other groups excluded outright: minus infinity instead of 0)."""
-    lf = logits.float()
+    lf = logits.float() if logit_bias is None else logits.float() + logit_bias.float()
     p = torch.softmax(lf, -1) if scoring == "softmax" else torch.sigmoid(lf)
     key = p + bias.float() if bias is not None else p.clone()
     if group_mode and n_group > 1:
@@ -642,7 +671,7 @@ def fp8_gemm(qa, sa, qw, sw, block: int, bias=None, out_dtype=torch.bfloat16):
     return out.to(out_dtype)
 
 
-def mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv=512, sinks=None):
+def mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv=512, sinks=None, window=-1):
     """Absorbed MLA: q [T, H, DK], cache [pages, 16, DK] -> out [T, H, dv] (values = the first dv
     latent dims).  ``sinks``: fp32 [H] logits joining each head's softmax denominator."""
     T, H, DK = q.shape
@@ -654,6 +683,8 @@ def mla_attn(q, cache, block_tables, tok_row, kv_lens, scale, dv=512, sinks=None
         pages = block_tables[int(tok_row[t])][: -(-L // P)].long()
         kv = flat[pages].reshape(-1, DK)[:L].float()
         s = (q[t].float() @ kv.t()) * scale
+        if window > 0 and L > window:
+            s[:, :L - window] = float("-inf")
         sk = None if sinks is None else sinks.float().view(H, 1)
         out[t] = (_softmax_sink(s, sk) @ kv[:, :dv]).to(q.dtype)
     return out
@@ -682,8 +713,8 @@ def conv_mix(x, w, state, cu, slot, reset, out):
             continue
         st = state[int(slot[s])]                                      # [C, K-1]
         prev = torch.zeros_like(st) if int(reset[s]) else st
-        seq = torch.cat([prev.t(), x[r0:r1]], 0)                      # [K-1+L, C] fp32
-        acc = x[r0:r1].clone()
+        seq = torch.cat([prev.t(), x[r0:r1].float()], 0)              # [K-1+L, C] fp32
+        acc = x[r0:r1].float().clone()
         for j in range(K):
             acc += wf[:, j] * seq[j:j + r1 - r0]
         out[r0:r1] = acc.to(out.dtype)
@@ -765,7 +796,7 @@ def row_norm(x, w, b, eps, kind):
     return n.to(w.dtype)
 
 
-def shift_norm(res, w, eps, x1, s1, x2, s2, w_offset, shift, state, seqs, out_dtype):
+def shift_norm(res, w, eps, x1, s1, x2, s2, w_offset, shift, state, seqs, out_dtype, bias=None):
     """``v = res + s1 x1 + s2 x2``; ``n = rmsnorm(v) (w_offset + w)``; with ``shift`` every row moves
     towards the row before it, ``n[t] + (n[t-1] - n[t]) shift`` (the row before a sequence's first:
     ``state[slot]``, zeros after a reset; the sequence's last n replaces it).  Returns (v, out)."""
@@ -774,6 +805,8 @@ def shift_norm(res, w, eps, x1, s1, x2, s2, w_offset, shift, state, seqs, out_dt
         v += float(s1) * x1.float()
     if x2 is not None:
         v += float(s2) * x2.float()
+    if bias is not None:
+        v += bias.float()
     n = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * (float(w_offset) + w.float())
     if shift is None:
         return v, n.to(out_dtype or w.dtype)
