@@ -340,3 +340,11 @@ def write_model(folder, cfg, weights):
         json.dump(cfg, f)
     save_file({k: v.contiguous() for k, v in weights.items()}, os.path.join(folder, "model.safetensors"))
     return folder
+
+
+def router_margin(cfg, weights, tokens):
+    """Smallest gap between the last chosen and the first unchosen router logit over all routed
+    evaluations of a prompt (infinite when every expert is always chosen)."""
+    m = [math.inf]
+    forward(cfg, weights, tokens, margins=m)
+    return m[0]

@@ -1,0 +1,148 @@
+"""Nivasun on the CPU path (fp32 reference ops) against the slow oracle: every mechanism alone,
+then whole models through the engine's replay entry -- whole prompts, prefill + token-by-token
+decoding, portions down to two tokens, batches of unequal requests, reused state slots and pages,
+planted keys at the window's edge, far back and at page borders -- and greedy generation through
+the scheduler."""
+import os
+import sys
+
+import pytest
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+import nivasun_cases as nc  # noqa: E402
+import nivasun_oracle as no  # noqa: E402
+from ome_amd.models.config import ModelConfig  # noqa: E402
+
+DEV, DT = "cpu", torch.float32
+KINDS = ["attention", "attention_2", "latent_attention"]
+
+
+def test_oracle_sanity():
+    nc.constants_matter_case()
+
+
+def test_config_envelope():
+    cfg = ModelConfig.from_hf(nc.config_a())
+    assert cfg.num_layers == 8 and cfg.architecture == "Nivasun"      # 1 + 3 x 2 + 1 layer runs
+    assert cfg.num_heads == 8 and cfg.num_kv_heads == 1               # two maps per head count as heads
+    assert [(i, p) for i, p, _ in no.run_order(nc.config_a())] == [(0, 0), (1, 0), (2, 0), (1, 1), (2, 1), (1, 2),
+                                                                   (2, 2), (3, 0)]
+
+
+def test_pair_embedding():
+    nc.pair_embedding_case(DEV, DT)
+    nc.pair_embedding_case(DEV, DT, W=7, V=300, buckets=1, mul_prev=1000003, mul_cur=999983, seed=8)
+
+
+@pytest.mark.parametrize("W,taps", [(40, 3), (7, 2), (24, 5), (16, 1)])
+def test_stream_norm_and_convolution(W, taps):
+    nc.stream_case(DEV, DT, W=W, taps=taps)
+
+
+def test_diff_head_norm():
+    nc.diff_head_norm_case(DEV, DT)
+    nc.diff_head_norm_case(DEV, DT, T=3, G=1, R=1, D=128, vdim=70, lam=-0.4, scale=1.0)
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(heads=1, kv_heads=1, dim=8, rot_dims=8),
+                                dict(heads=3, kv_heads=3, dim=10, window=1000, rot_dims=0, scale=1.3),
+                                dict(heads=4, kv_heads=1, dim=70, window=3, rot_dims=6, base=5000.0),
+                                dict(heads=2, kv_heads=2, dim=6, window=1, rot_dims=6)])
+def test_key_valued_attention_alone(kw):
+    nc.mixer_alone(DEV, DT, no.keyed_layer(**kw))
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(heads=1, kv_heads=1, dim=8, vdim=8, window=1000, rot_dims=8, diff=0.0),
+                                dict(heads=4, kv_heads=1, dim=5, vdim=7, window=6, rot_dims=2, scale=0.9, diff=0.8),
+                                dict(heads=2, kv_heads=2, dim=36, vdim=70, window=1, rot_dims=0),
+                                dict(heads=18, kv_heads=9, dim=4, vdim=2, window=20)])
+def test_differential_attention_alone(kw):
+    nc.mixer_alone(DEV, DT, no.diff_layer(**kw))
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(heads=1, dim=8, vdim=8, kv_rank=8, q_rank=8, window=1000),
+                                dict(heads=5, dim=4, vdim=12, kv_rank=70, q_rank=3, window=2, scale=0.7),
+                                dict(heads=18, dim=6, vdim=4, kv_rank=16, q_rank=9, window=20),
+                                dict(heads=2, dim=12, vdim=6, kv_rank=130, q_rank=40, window=1)])
+def test_latent_attention_alone(kw):
+    nc.mixer_alone(DEV, DT, no.latent_layer(**kw))
+
+
+def test_feed_forward_alone():
+    for f, width in ((no.moe(), 24), (no.moe(6, 3, 9, 0), 24), (no.moe(2, 2, 8, 0), 24), (no.moe(1, 1, 8, 5), 24),
+                     (no.moe(8, 3, 32, 32), 64)):
+        assert not nc.moe_case(DEV, DT, f, width)
+    nc.router_bias_case(DEV)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_window_edge(kind):
+    for cuts in ([60], [55] + [1] * 5, [16, 16, 16, 12], nc.portions(60, [2, 3, 7])):
+        nc.planted_window_case(DEV, DT, kind, 8, True, cuts)       # the last key inside the window
+        nc.planted_window_case(DEV, DT, kind, 9, False, cuts)      # the first one outside
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_far_key_and_page_borders(kind):
+    for back in (300, 303, 304, 319):                              # keys 131 / 128 / 127 / 112 of 432 rows
+        nc.planted_far_case(DEV, DT, kind, 432, back, [400] + [1] * 32)
+    nc.planted_far_case(DEV, DT, kind, 432, 415, nc.portions(432, [64, 35, 2, 17]))   # key 16, in portions
+
+
+# ------------------------------------------------------------------------------ whole models
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, cfg in (("a", nc.config_a()), ("b", nc.config_b()), ("c", nc.config_c())):
+        w = no.make_weights(cfg, seed=11)
+        out[name] = (cfg, w, no.write_model(str(tmp_path_factory.mktemp("niv_" + name)), cfg, w), {})
+    return out
+
+
+@pytest.mark.parametrize("name", ["a", "b", "c"])
+def test_schedules_match_oracle(models, name):
+    cfg, w, path, cache = models[name]
+    toks = dict(zip("pqrstu", nc.prompts(cfg, w, [1, 2, 37, 70, 16, 33], min_margin=1e-4)))
+    eng = nc.make_engine(path, DEV, "float32", max_tokens=192)
+    for sched in (nc.whole_schedule(toks), nc.decode_schedule(toks, 24),
+                  nc.chunked_schedule(toks, [2, 3, 17, 1, 32, 2]), nc.mixed_schedule(toks, [1, 2, 5, 16, 1, 31])):
+        nc.assert_matches_oracle(eng, cfg, w, toks, sched, 2e-4, cache)
+
+
+def test_slots_and_pages_are_reused(models):
+    cfg, w, path, cache = models["a"]
+    ps = nc.prompts(cfg, w, [20, 3, 41, 17, 2, 33, 9, 48, 1, 25], seed=5, min_margin=1e-4)
+    toks = {f"r{i}": t for i, t in enumerate(ps)}
+    eng = nc.make_engine(path, DEV, "float32", max_tokens=160)
+    nc.assert_matches_oracle(eng, cfg, w, toks, nc.mixed_schedule(toks, [2, 7, 1, 16, 3], seed=8), 2e-4, cache)
+    assert eng.runner.pages.num_free == eng.runner.pages.num_pages - 1 and not eng.scheduler.running
+
+
+def test_long_decoding(models):
+    """Eighty tokens one by one: every window of the stack passes over decoded tokens only."""
+    cfg, w, path, cache = models["a"]
+    toks = {"x": nc.prompts(cfg, w, [100], seed=9, min_margin=1e-4)[0]}
+    eng = nc.make_engine(path, DEV, "float32", max_tokens=128)
+    nc.assert_matches_oracle(eng, cfg, w, toks, nc.decode_schedule(toks, 80), 2e-4, cache)
+
+
+def test_greedy_generation(models):
+    cfg, w, path, _ = models["a"]
+    ps = nc.prompts(cfg, w, [5, 19, 1], seed=13)
+    eng = nc.make_engine(path, DEV, "float32", max_tokens=256)
+    got = nc.greedy_engine(eng, ps, 10)
+    for p, g in zip(ps, got):
+        want, gap = nc.greedy_reference(cfg, w, p, 10)
+        assert len(g) == 10
+        if gap > 1e-3:                 # only clear-cut argmaxes are pinned
+            assert g == want
+
+
+def test_incomplete_checkpoint_is_refused(models, tmp_path):
+    cfg, w, _, _ = models["a"]
+    for gone in ("l0.mix.lq2", "l1.mix.temp", "bigram", "loop.step", "l2.mix.g", "l0.mlp.router.b"):
+        path = no.write_model(str(tmp_path / gone), cfg, {k: v for k, v in w.items() if k != gone})
+        with pytest.raises(ValueError, match=gone.split(".")[-1]):
+            nc.make_engine(path, DEV, "float32")
