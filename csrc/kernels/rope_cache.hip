@@ -329,16 +329,18 @@ __global__ __launch_bounds__(256) void wide_norm_rope_cache_kernel(
 }
 
 // The same op with 16-byte accesses, for the shapes real layers have: interleaved rotation (a
-// pair never leaves its 8-wide vector), dim % 8 == 0, rows and pointers 16-byte aligned.  A unit
-// is one 8-dim vector of one head; pass one sums the squares from vector loads, pass two re-reads
-// the (cache-hot) row, normalises, rotates in registers and stores one vector.
+// pair never leaves its 8-wide vector) or half-split pairs with rot_dim % 16 == 0 (the partner is
+// the vector rot_dim / 2 further or nearer, read as a second vector), dim % 8 == 0, rows and
+// pointers 16-byte aligned.  A unit is one 8-dim vector of one head; pass one sums the squares from
+// vector loads, pass two re-reads the (cache-hot) row, normalises, rotates in registers and stores
+// one vector.
 __global__ __launch_bounds__(256) void wide_norm_rope_cache_vec_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k, int64_t k_stride,
     const bf16* __restrict__ v, int64_t v_stride, const int* __restrict__ positions,
     const float* __restrict__ cos_sin, int rot_dim, const bf16* __restrict__ qn_w, const bf16* __restrict__ kn_w,
     float eps, bf16* __restrict__ q_out, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
     const int* __restrict__ slots, int Hq, int Hkv, int dim, int vdim, int D, int P,
-    const float* __restrict__ q_scale, int v_rep) {
+    const float* __restrict__ q_scale, int v_rep, int interleaved) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
   const bf16* qr = q + t * q_stride;
@@ -389,14 +391,35 @@ __global__ __launch_bounds__(256) void wide_norm_rope_cache_vec_kernel(
 #pragma unroll
         for (int j = 0; j < 8; ++j) f[j] = (float)x[j];
       }
+      if (interleaved) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int d = d0 + 2 * j;
-        if (d < rot_dim) {
-          const float c = cs[d >> 1], sn = cs[half + (d >> 1)];
-          const float a = f[2 * j], b = f[2 * j + 1];
-          f[2 * j] = a * c - b * sn;
-          f[2 * j + 1] = b * c + a * sn;
+        for (int j = 0; j < 4; ++j) {
+          const int d = d0 + 2 * j;
+          if (d < rot_dim) {
+            const float c = cs[d >> 1], sn = cs[half + (d >> 1)];
+            const float a = f[2 * j], b = f[2 * j + 1];
+            f[2 * j] = a * c - b * sn;
+            f[2 * j + 1] = b * c + a * sn;
+          }
+        }
+      } else if (d0 < rot_dim) {   // half-split: dim d pairs with d + half (d < half) or d - half
+        const bool lowh = d0 < half;
+        const int dp = lowh ? d0 + half : d0 - half, a0 = lowh ? d0 : dp;
+        const bf16x8 y = ld8(src - d0 + dp);
+        float pv[8];
+        if (nw != nullptr) {
+          const bf16x8 wv = ld8(nw + hh * dim + dp);
+          const float rs = is_q ? rq : rk;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pv[j] = (float)y[j] * rs * (float)wv[j];
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) pv[j] = (float)y[j];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float c = cs[a0 + j], sn = cs[half + a0 + j];
+          f[j] = lowh ? f[j] * c - pv[j] * sn : f[j] * c + pv[j] * sn;
         }
       }
       const float qs = is_q && q_scale != nullptr ? q_scale[hh] : 1.f;
@@ -432,7 +455,8 @@ OME_API int ome_wide_norm_rope_cache(const void* q, int64_t q_stride, const void
     OME_CHECK_LAUNCH();
     return 0;
   }
-  const bool vec = interleaved && dim % 8 == 0 && D % 8 == 0 && q_stride % 8 == 0 && k_stride % 8 == 0 &&
+  const bool vec = (interleaved || rot_dim % 16 == 0) && dim % 8 == 0 && D % 8 == 0 && q_stride % 8 == 0 &&
+                   k_stride % 8 == 0 &&
                    (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)q_out % 16 == 0 &&
                    (uintptr_t)k_cache % 16 == 0 && (qn_w == nullptr || (uintptr_t)qn_w % 16 == 0) &&
                    (kn_w == nullptr || (uintptr_t)kn_w % 16 == 0);
@@ -440,7 +464,7 @@ OME_API int ome_wide_norm_rope_cache(const void* q, int64_t q_stride, const void
     wide_norm_rope_cache_vec_kernel<<<T, 256, 0, stream>>>(
         (const bf16*)q, q_stride, (const bf16*)k, k_stride, (const bf16*)v, v_stride, positions, cos_sin, rot_dim,
         (const bf16*)qn_w, (const bf16*)kn_w, eps, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, slots, Hq, Hkv, dim,
-        vdim, D, P, q_scale, v_rep);
+        vdim, D, P, q_scale, v_rep, interleaved);
     OME_CHECK_LAUNCH();
     return 0;
   }

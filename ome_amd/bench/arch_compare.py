@@ -1,5 +1,10 @@
 """Layer-list designs beside their closest existing model at equal size (``bench.py --arch-compare
-[--arch-design zavilorn|metitar|milenex]``).
+[--arch-design zavilorn|metitar|milenex|nivasun]``).
+
+Nivasun (parallel blocks: one norm feeding a mixer -- differential, key-valued or windowed latent
+attention behind a short convolution -- and a biased-router mixture of SiLU-GLU experts with a gated
+shared expert, on a hashed token-pair embedding) stands beside the same GPT-OSS-style stack of the
+same width, depth, effective head counts, window and expert sizes.
 
 Milenex (token shift, sliding-window attention with sinks: one kind with short convolutions, rotary
 pairs and unit-RMS q / k, one with a logarithmic distance bias and weights mixed across heads;
@@ -117,6 +122,27 @@ def milenex_config(s: dict, window: int = 1024) -> dict:
     layers = [{"type": "attention_2", "mixer": dict(base), "mlp": moe}, {"type": "attention", "mixer": rot, "mlp": moe}] * 4
     return {"architecture": "Milenex", "layers": layers, "norm": {"eps": 1e-6}, "vocab": s["vocab"],
             "width": s["width"], "max_positions": 8192}
+
+
+def nivasun_config(s: dict, window: int = 1024) -> dict:
+    """[differential, key-valued, differential, latent] x 2 with 128-wide heads (the differential
+    layers have half the heads, each with two score maps), a 256-wide latent, 4 taps in front of every
+    mixer, every layer with 32 experts, top 4, and a gated shared expert of an expert's width."""
+    moe = {"kind": "moe", "router": {"experts": s["experts"], "top": s["top"]}, "expert": {"ff": s["eff"]},
+           "shared": {"ff": s["eff"]}}
+    mask, rot = {"size": window}, {"base": 10000.0, "dims": 64}
+    dif = {"type": "attention_2", "mlp": moe,
+           "mixer": {"heads": s["heads"] // 2, "kv_heads": s["kv"] // 2, "dim": 128, "vdim": 128, "mask": mask, "rot": rot,
+                     "scale": 128 ** -0.5, "diff": 0.5}}
+    key = {"type": "attention", "mlp": moe,
+           "mixer": {"heads": s["heads"], "kv_heads": s["kv"], "dim": 128, "vdim": 128, "mask": mask, "rot": rot,
+                     "scale": 128 ** -0.5}}
+    lat = {"type": "latent_attention", "mlp": moe,
+           "mixer": {"heads": s["heads"], "dim": 128, "vdim": 128, "kv_rank": 256, "q_rank": 768, "mask": mask,
+                     "scale": 128 ** -0.5}}
+    return {"architecture": "Nivasun", "layers": [dif, key, dif, lat] * 2, "norm": {"eps": 1e-6}, "vocab": s["vocab"],
+            "width": s["width"], "max_positions": 8192, "canon": {"taps": 4}, "logit_softcap": 30.0,
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 36313, "mul_cur": 27191}}}
 
 
 def gpt_oss_like_config(s: dict, window: int = 1024) -> dict:
@@ -514,8 +540,169 @@ def kernel_table_milenex(T: int = 4096, B: int = 64, ctx: int = 4096, width: int
     return rows
 
 
+def kernel_table_nivasun(T: int = 4096, B: int = 64, ctx: int = 4096, width: int = 4096) -> list[dict]:
+    """Nivasun's kernels beside their like kernels (same columns as :func:`kernel_table`)."""
+    from ome_amd import ops
+    from ome_amd.models.config import plain_rope_table
+    from ome_amd.models.mixers import GroupRoutedMoE
+
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def pair(name, new, like, bytes_new, bytes_like, note="", iters=30):
+        tn, tl = _time_us(new, iters), _time_us(like, iters)
+        fn, fl = bytes_new / tn / 1e3 / HBM_GBS, bytes_like / tl / 1e3 / HBM_GBS
+        rows.append({"kernel": name, "us": round(tn, 1), "roofline": round(fn, 3), "like_us": round(tl, 1),
+                     "like_roofline": round(fl, 3), "vs_like": round(fl / max(fn, 1e-9), 2), "note": note})
+
+    def seqs(lens):
+        cu = torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32, device=dev)
+        n = len(lens)
+        return cu, torch.arange(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev)
+
+    torch.manual_seed(0)
+    Hq, Hkv, D, P, W = 32, 8, 128, 16, 1024
+    for R, tag, lens in ((T, "prefill", [T // 8] * 8), (B, "decode", [1] * B)):
+        sq = seqs(lens)
+        # ---- token-pair embedding vs the plain embedding
+        V = 32768
+        ids = torch.randint(0, V, (R,), dtype=torch.int32, device=dev)
+        emb, prs = torch.randn(V, width, device=dev).to(bf), torch.randn(65522, width, device=dev).to(bf)
+        prev = torch.zeros(len(lens) + 1, dtype=torch.int32, device=dev)
+        pair(f"pair_embedding_f32 ({tag})",
+             lambda: ops.pair_embedding_f32(ids, emb, 1.0, prs, 65521, 36313, 27191, prev, sq),
+             lambda: ops.embedding(ids, emb), R * width * 8, R * width * 4,
+             "two table rows in, an fp32 row out: 8 B / element against 4")
+        # ---- stream update with two addends and a pass vector + single-gain norm vs add + RMSNorm on a bf16 stream
+        res = torch.randn(R, width, device=dev)
+        y1, y2 = torch.randn(R, width, device=dev).to(bf), torch.randn(R, width, device=dev).to(bf)
+        w, step = torch.ones(width, device=dev, dtype=bf), torch.randn(width, device=dev).to(bf)
+        rb, xb = res.to(bf), y1.clone()
+        pair(f"shift_norm, two addends + pass vector ({tag})",
+             lambda: ops.shift_norm(res, w, 1e-6, y1, 1.0, y2, 1.0, out_dtype=bf, bias=step),
+             lambda: ops.fused_add_rmsnorm(xb, rb, w, 1e-6), R * width * 14, R * width * 8,
+             "fp32 stream + two sublayer outputs: 14 B / element against 8")
+        # ---- residual convolution of the normed rows vs the causal conv of the recurrent mixers
+        h = torch.randn(R, width, device=dev).to(bf)
+        cw = (torch.randn(width, 4, device=dev) * 0.3).to(bf)
+        st32 = torch.zeros(len(lens), width, 3, device=dev)
+        stb = torch.zeros(len(lens), width, 3, device=dev, dtype=bf)
+        pair(f"conv_mix 4 taps on normed rows ({tag})", lambda: ops.conv_mix(h, cw, st32, *sq, bf),
+             lambda: ops.ssm_conv1d(h, cw, None, stb, *sq), R * width * 4, R * width * 4,
+             "like: the depthwise conv + SiLU of Mamba-2 / delta-rule inputs")
+        # ---- rotary + temperature + keys stored as values / values shared by two key heads vs Qwen3's prep
+        n_pages = R // P + 2
+        kc = torch.zeros(n_pages, Hkv, P, D, device=dev, dtype=bf)
+        vc = torch.zeros(n_pages, Hkv, D, P, device=dev, dtype=bf)
+        C = (Hq + 2 * Hkv) * D
+        qkv = torch.randn(R, C, device=dev).to(bf)
+        pos = torch.arange(R, dtype=torch.int32, device=dev) % 2048
+        slots = torch.arange(R, dtype=torch.int32, device=dev) + P
+        cs = plain_rope_table(10000.0, 64, 2049, dev)
+        qo = torch.empty(R, Hq, D, device=dev, dtype=bf)
+        hn = torch.ones(D, device=dev, dtype=bf)
+        temp = torch.rand(Hq, device=dev) + 0.5
+        qv, kv_ = qkv[:, :Hq * D], qkv[:, Hq * D:(Hq + Hkv) * D]
+        like = lambda: ops.rope_qkv_cache(qkv, pos, cs, 64, qo, kc, vc, slots, Hq, Hkv, D, True, hn, hn, 1e-6)   # noqa: E731
+        pair(f"wide_norm_rope_cache, half-split pairs + temperature, v = k ({tag})",
+             lambda: ops.wide_norm_rope_cache(qv, kv_, kv_, pos, cs, 64, False, None, None, 0.0, qo, kc, vc, slots, Hq,
+                                              Hkv, D, D, q_scale=temp),
+             like, R * ((Hq + Hkv) * D * 2 + (Hq + 2 * Hkv) * D * 2), R * C * 2 * 2,
+             "like: Qwen3's per-head norm + rotary + cache write")
+        vh = qkv[:, (Hq + Hkv) * D:(Hq + Hkv) * D + (Hkv // 2) * D]
+        pair(f"wide_norm_rope_cache, interleaved pairs, values under two key heads ({tag})",
+             lambda: ops.wide_norm_rope_cache(qv, kv_, vh, pos, cs, 64, True, None, None, 0.0, qo, kc, vc, slots, Hq,
+                                              Hkv, D, D, v_rep=2),
+             like, R * ((Hq + Hkv + Hkv // 2) * D * 2 + (Hq + 2 * Hkv) * D * 2), R * C * 2 * 2)
+        # ---- combine of the two maps + head norm vs the sigmoid head gate
+        a = torch.randn(R, Hq, D, device=dev).to(bf)
+        gate = torch.randn(R, Hq * D, device=dev).to(bf)
+        pair(f"diff_head_norm ({tag})", lambda: ops.diff_head_norm(a, 0.6, 1e-6, 0.5, 4, D),
+             lambda: ops.head_gate(a, gate, D, 0), R * Hq * D * 3, R * Hq * D * 6,
+             "reads 2 heads, writes 1; like: Zavilorn's output gate (reads 2, writes 1 per head)")
+        # ---- routed feed-forward: biased router + softmax over the chosen + gated shared expert vs GPT-OSS's experts
+        E, k, ff = 32, 4, 2048
+        moe = GroupRoutedMoE(width, E, k, ff, 0.0, 1, 1, ff, 0.0, dev, bf, act=0, renorm=True, router_bias=True,
+                             correction=False)
+        moe.init_random(torch.Generator(device=dev).manual_seed(1), 0.02)
+        x = torch.randn(R, width, device=dev).to(bf)
+        lg = torch.randn(R, E, device=dev)
+        tw, tid = ops.moe_route(lg, k, True, "softmax")
+        touched = min(E, R * k) * 3 * ff * width * 2
+        pair(f"biased-router moe 32 experts top 4 + shared ({tag})", lambda: moe.forward(x),
+             lambda: ops.fused_moe(x, tw, tid, moe.w13, moe.w2, 2, 1.0), touched + 3 * ff * width * 2, touched,
+             "new: router GEMM + route + shared expert (3 GEMMs) + grouped GEMMs + combine; like: grouped GEMMs + combine",
+             10)
+    # ---- decode over a long context, window 1024
+    per = ctx // P
+    kc = (torch.randn(B * per + 1, Hkv, P, D, device=dev) * 0.3).to(bf)
+    vc = (torch.randn(B * per + 1, Hkv, D, P, device=dev) * 0.3).to(bf)
+    bt = (torch.arange(B * per, dtype=torch.int32, device=dev) + 1).view(B, per)
+    sl = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+    q = (torch.randn(B, Hq, D, device=dev) * 0.3).to(bf)
+    sinks = torch.zeros(Hq, device=dev)
+    ws = ops.DecodeWorkspace(B, Hq, D, ctx, 0, dev, parts=4)
+    kvb = B * Hkv * D * 2 * 2 * W
+    like_dec = lambda: ops.paged_decode(q, kc, vc, bt, sl, 0.09, ws, W, sinks=sinks)   # noqa: E731
+    pair("differential attention decode 64 x 4096 ctx: 16 heads x 2 maps over 4 x 2 key heads + combine",
+         lambda: ops.diff_head_norm(ops.paged_decode(q, kc, vc, bt, sl, 0.09, ws, W), 0.6, 1e-6, 0.5, 4, D), like_dec,
+         B * (Hkv * D * 2 + (Hkv // 2) * D * 2) * W, kvb,
+         "the values of a kv group sit under both of its key heads: 4/3 of the bytes that must move", 10)
+    pair("key-valued attention decode (sinks, temperature folded into q): the like kernel's own launch",
+         like_dec, like_dec, kvb, kvb, "", 10)
+    R_, H_ = 256, 32
+    DK, DV = ops.latent_shape(R_, 0)
+    lc = (torch.randn(B * per + 1, P, DK, device=dev) * 0.3).to(bf)
+    ql = (torch.randn(B, H_, DK, device=dev) * 0.3).to(bf)
+    rows_i = torch.arange(B, dtype=torch.int32, device=dev)
+    slw = torch.full((B,), W, dtype=torch.int32, device=dev)
+    mws = ops.MLAWorkspace(dev)
+    pair("latent attention decode, window 1024 of 4096 ctx (288-wide rows)",
+         lambda: ops.latent_attn(ql, lc, bt, rows_i, sl, 0.09, DV, mws, window=W),
+         lambda: ops.latent_attn(ql, lc, bt, rows_i, slw, 0.09, DV, mws), B * W * DK * 2, B * W * DK * 2,
+         "like: the same kernel without a window over a 1024-token context", 10)
+    # ---- prefill, 2 x 2048 rows
+    q_lens = [2048, 2048]
+    Tq = sum(q_lens)
+    qp = (torch.randn(Tq, Hq, D, device=dev) * 0.3).to(bf)
+    cu = torch.tensor([0, 2048, 4096], dtype=torch.int32, device=dev)
+    kl = torch.tensor(q_lens, dtype=torch.int32, device=dev)
+    bt2 = (torch.arange(2 * 128, dtype=torch.int32, device=dev) + 1).view(2, 128)
+    items = torch.tensor(ops.prefill_work_items(q_lens, q_lens), dtype=torch.int32, device=dev)
+    flops = 4.0 * Hq * D * sum(min(W, i + 1) for i in range(2048)) * 2
+    tn = _time_us(lambda: ops.diff_head_norm(ops.paged_prefill(qp, kc, vc, bt2, cu, kl, items, 0.09, W), 0.6, 1e-6, 0.5,
+                                             4, D), 5)
+    tl = _time_us(lambda: ops.paged_prefill(qp, kc, vc, bt2, cu, kl, items, 0.09, W, sinks=sinks), 5)
+    rows.append({"kernel": "differential attention prefill 2 x 2048 rows, window 1024 (+ combine)", "us": round(tn, 1),
+                 "roofline": round(flops / tn / 1e6 / 2.5e3, 3), "like_us": round(tl, 1),
+                 "like_roofline": round(flops / tl / 1e6 / 2.5e3, 3), "vs_like": round(tn / tl, 2),
+                 "note": "share of 2.5 PFLOP/s bf16 (q.k and p.v only); like: the MFMA sliding-window kernel with sinks"})
+    qlp = (torch.randn(Tq, H_, DK, device=dev) * 0.3).to(bf)
+    tok_row = torch.arange(Tq, dtype=torch.int32, device=dev) // 2048
+    lens_p = (torch.arange(Tq, dtype=torch.int32, device=dev) % 2048) + 1
+    lflops = 2.0 * H_ * (DK + DV) * 2
+    tn = _time_us(lambda: ops.latent_attn(qlp, lc, bt2, tok_row, lens_p, 0.09, DV, mws, window=W), 5)
+    tl = _time_us(lambda: ops.latent_attn(qlp, lc, bt2, tok_row, lens_p, 0.09, DV, mws), 5)
+    fw, fa = lflops * sum(min(W, i + 1) for i in range(2048)), lflops * sum(i + 1 for i in range(2048))
+    rows.append({"kernel": "latent attention prefill 2 x 2048 rows, window 1024", "us": round(tn, 1),
+                 "roofline": round(fw / tn / 1e6 / 2.5e3, 3), "like_us": round(tl, 1),
+                 "like_roofline": round(fa / tl / 1e6 / 2.5e3, 3), "vs_like": round((fa / tl) / (fw / tn), 2),
+                 "note": "like: the same kernel without a window (all 2048 keys); both as share of 2.5 PFLOP/s"})
+    return rows
+
+
 def run(sizes=("2k", "4k"), kernels: bool = True, only: str | None = None, design: str = "zavilorn") -> dict:
     out = {"throughput": [], "kernels": []}
+    if design == "nivasun":
+        for k in sizes:
+            s = X_SIZES[k]
+            if only in (None, "nivasun"):
+                out["throughput"].append(throughput(f"nivasun-{k}", nivasun_config(s)))
+            if only in (None, "gpt-oss"):
+                out["throughput"].append(throughput(f"gpt-oss-like-{k}", gpt_oss_like_config(s)))
+        if kernels:
+            out["kernels"] = kernel_table_nivasun()
+        return out
     if design == "milenex":
         for k in sizes:
             s = X_SIZES[k]
@@ -553,9 +740,10 @@ def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--sizes", default="2k,4k")
     ap.add_argument("--no-kernels", action="store_true")
-    ap.add_argument("--only", choices=["zavilorn", "nemotron", "metitar", "deepseek", "milenex", "gpt-oss"], default=None,
+    ap.add_argument("--only", choices=["zavilorn", "nemotron", "metitar", "deepseek", "milenex", "gpt-oss", "nivasun"],
+                    default=None,
                     help="one stack (for kernel traces)")
-    ap.add_argument("--design", choices=["zavilorn", "metitar", "milenex"], default="zavilorn")
+    ap.add_argument("--design", choices=["zavilorn", "metitar", "milenex", "nivasun"], default="zavilorn")
     ap.add_argument("--no-throughput", action="store_true", help="the kernel table only")
     a = ap.parse_args(argv)
     res = run(() if a.no_throughput else tuple(a.sizes.split(",")), not a.no_kernels, a.only, a.design)

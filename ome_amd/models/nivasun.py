@@ -134,6 +134,10 @@ class NivasunForCausalLM(LlamaForCausalLM):
         self.kv_dims_per_layer = {r: b.D for r, b in shape.items()}
         # (a latent layer's key rows carry their values: no value array)
         self.kv_value_dim = {r: 0 if isinstance(b, LatentAttention) and b.latent_cache else b.D for r, b in shape.items()}
+        # fewest kv heads among the layers that run the split-K decode kernel (latent layers on the latent
+        # kernel bring their own workspace): the runner partitions its decode workspace by it
+        paged = [self.kv_heads_per_layer[r] for r, b in shape.items() if not (isinstance(b, LatentAttention) and b.latent_cache)]
+        self.decode_ws_kv_heads = min(paged) if paged else None
 
     def _share_passes(self) -> None:
         """Blocks of later passes: the first pass's weights, their own cache layer."""

@@ -344,7 +344,8 @@ class ModelRunner:
         key = bs if not half else (bs, half)
         ws = self._ws_cache.get(key)
         if ws is None:
-            hkv = self.model.tp.hkv
+            # (a model whose split-K decode layers all have more kv heads than its envelope says so)
+            hkv = getattr(self.model, "decode_ws_kv_heads", None) or self.model.tp.hkv
             parts = max(1, math.ceil(1024 / max(1, bs * hkv)))
             span = self.max_context + self.P  # seq_lens never exceed this: one part covers it all
             if parts > 1 and os.environ.get("OME_DECODE_DYN_PARTS", "1") == "1":
