@@ -45,11 +45,10 @@ def causal_conv(u, w):
     """y_t = sum_j w[:, j] u_{t - K + 1 + j}, rows before the start are zero; u [T, C], w [C, K]."""
     T, K = u.shape[0], w.shape[1]
     y = torch.zeros_like(u)
-    for t in range(T):
-        for j in range(K):
-            s = t - K + 1 + j
-            if s >= 0:
-                y[t] += w[:, j] * u[s]
+    for j in range(K):
+        back = K - 1 - j                      # tap j reads the row `back` steps before
+        if back < T:
+            y[back:] += w[:, j] * u[:T - back]
     return y
 
 
@@ -174,9 +173,11 @@ def moe_ff(h, w, f):
     val, idx = z.topk(top, -1)
     p = torch.softmax(val, -1)
     y = torch.zeros_like(h)
-    for t in range(h.shape[0]):
-        for j in range(top):
-            y[t] += p[t, j] * glu_expert(h[t:t + 1], w, f"e{int(idx[t, j])}.")[0]
+    for e in range(f["router"]["experts"]):
+        share = (p * (idx == e)).sum(-1, keepdim=True)        # the token's weight for expert e, 0 if not chosen
+        rows = share[:, 0] > 0
+        if rows.any():
+            y[rows] += share[rows] * glu_expert(h[rows], w, f"e{e}.")
     if f.get("shared"):
         y = y + glu_expert(h, w, "shared.") * sigmoid(h @ w["shared.sg"].T)
     return y
