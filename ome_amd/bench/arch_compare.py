@@ -141,7 +141,7 @@ def nivasun_config(s: dict, window: int = 1024) -> dict:
            "mixer": {"heads": s["heads"], "dim": 128, "vdim": 128, "kv_rank": 256, "q_rank": 768, "mask": mask,
                      "scale": 128 ** -0.5}}
     return {"architecture": "Nivasun", "layers": [dif, key, dif, lat] * 2, "norm": {"eps": 1e-6}, "vocab": s["vocab"],
-            "width": s["width"], "max_positions": 8192, "canon": {"taps": 4}, "logit_softcap": 30.0,
+            "width": s["width"], "max_positions": 8192, "canon": {"taps": 4}, "logit_softcap": 25.0,
             "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 36313, "mul_cur": 27191}}}
 
 

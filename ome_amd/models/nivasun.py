@@ -169,7 +169,7 @@ class NivasunForCausalLM(LlamaForCausalLM):
     def alloc_state(self, slots: int) -> None:
         for b in self.mix.values():
             b.alloc_state(slots)
-        if self.taps > 1:
+        if self.taps:
             for r in range(len(self.runs)):
                 self.conv_state[r] = torch.zeros(slots, self.cfg.hidden_size, self.taps - 1, dtype=torch.float32,
                                                  device=self.device)
@@ -281,8 +281,7 @@ class NivasunForCausalLM(LlamaForCausalLM):
         for r, (i, p) in enumerate(self.runs):
             step = self.loop_step[p] if self.looped and i == self.loop_start else None
             x, h = ops.shift_norm(x, self.ln1[i], eps, y1, 1.0, y2, 1.0, out_dtype=dt, bias=step)
-            hm = ops.conv_mix(h, self.canon[i], self.conv_state[r], cu, slot, reset, dt) if self.taps > 1 else \
-                (h if not self.taps else (h.float() * (1.0 + self.canon[i].float()[:, 0])).to(dt))
+            hm = ops.conv_mix(h, self.canon[i], self.conv_state[r], cu, slot, reset, dt) if self.taps else h
             y1 = self.mix[r].forward(hm, ctx)
             y2 = self.ff[i].forward(h) if i in self.ff else None
             if dbg is not None:

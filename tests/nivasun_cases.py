@@ -233,20 +233,18 @@ def stream_case(dev, dt, W=40, taps=3, seed=5):
         r, h = ops.shift_norm(x, gain.expand(W).contiguous().to(dev), EPS, cat(y1), 1.0, cat(y2), 1.0, out_dtype=dt,
                               bias=bias.to(dev))
         assert r.data_ptr() == x.data_ptr()
-        hc = ops.conv_mix(h, cw.to(dev), state, cu, slot, reset, dt) if taps > 1 else None
+        hc = ops.conv_mix(h, cw.to(dev), state, cu, slot, reset, dt)
         a = 0
         for s in live:
             assert rel(r[a:a + lens[s]], v64[s][off[s]:off[s] + lens[s]]) < 1e-6
             got_h[s].append(h[a:a + lens[s]].cpu())
-            if hc is not None:
-                got_c[s].append(hc[a:a + lens[s]].cpu())
+            got_c[s].append(hc[a:a + lens[s]].cpu())
             a += lens[s]
     for s in range(3):
         h = torch.cat(got_h[s])
         assert rel(h, h64[s]) < (0.02 if dt == BF else 1e-5), s
-        if taps > 1:   # the convolution reads the rounded rows
-            hq = h.to(F64)
-            assert rel(torch.cat(got_c[s]), hq + no.causal_conv(hq, cw.to(F64))) < (0.02 if dt == BF else 1e-5), s
+        hq = h.to(F64)        # the convolution reads the rounded rows
+        assert rel(torch.cat(got_c[s]), hq + no.causal_conv(hq, cw.to(F64))) < (0.02 if dt == BF else 1e-5), s
 
 
 def diff_head_norm_case(dev, dt, T=9, G=2, R=3, D=64, vdim=10, lam=0.7, scale=0.6, seed=4):
