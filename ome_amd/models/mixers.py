@@ -53,10 +53,28 @@ class MixerCtx:
     cache: dict = field(default_factory=dict)   # tensors derived once per step and shared by the layers
 
 
+MAX_HEAD_GROUP = 16   # query heads per kv head one launch of the paged attention kernels takes
+
+
 def paged_attention(q: torch.Tensor, k_cache, v_cache, meta: AttnMeta, scale: float, window: int = -1,
                     keep_first: int = 0, sinks: torch.Tensor | None = None) -> torch.Tensor:
     """Decode / prefill / mixed dispatch over the paged cache (q [T, Hq, D] -> [T, Hq, D]).
-    ``sinks``: fp32 [Hq] logits that join each head's softmax denominator (no key, no value)."""
+    ``sinks``: fp32 [Hq] logits that join each head's softmax denominator (no key, no value).
+    More than ``MAX_HEAD_GROUP`` query heads per kv head run as several launches over slices of
+    every kv head's group."""
+    T, Hq, D = q.shape
+    Hkv = k_cache.shape[1]
+    R = Hq // Hkv
+    if R > MAX_HEAD_GROUP and q.is_contiguous():
+        q4 = q.view(T, Hkv, R, D)
+        out = torch.empty_like(q4)
+        for c in range(0, R, MAX_HEAD_GROUP):
+            e = min(R, c + MAX_HEAD_GROUP)
+            sk = None if sinks is None else sinks.view(Hkv, R)[:, c:e].reshape(-1).contiguous()
+            part = paged_attention(q4[:, :, c:e].reshape(T, Hkv * (e - c), D).contiguous(), k_cache, v_cache, meta, scale, window,
+                                   keep_first, sk)
+            out[:, :, c:e] = part.view(T, Hkv, e - c, D)
+        return out.view(T, Hq, D)
     kw = dict(window=window, keep_first=keep_first, sinks=sinks)
     if meta.is_decode:
         return ops.paged_decode(q, k_cache, v_cache, meta.block_tables, meta.seq_lens, scale, meta.decode_ws,
@@ -788,8 +806,8 @@ class KeyValuedAttention(_Block):
     def __init__(self, layer: int, width: int, heads: int, kv_heads: int, dim: int, window: int, rot_base: float,
                  rot_dims: int, scale: float, max_positions: int, device, dtype, interleaved: bool = False):
         super().__init__(device, dtype)
-        if heads % kv_heads or heads // kv_heads > 16:
-            raise ValueError(f"attention: {heads} query heads over {kv_heads} kv heads (groups of <= 16 supported)")
+        if heads % kv_heads:
+            raise ValueError(f"attention: {heads} query heads do not divide over {kv_heads} kv heads")
         self.layer, self.width, self.Hq, self.Hkv, self.dim = layer, width, heads, kv_heads, dim
         self.window = int(window) if window and window > 0 else -1
         self.rot_dims, self.scale, self.interleaved = int(rot_dims), float(scale), bool(interleaved)
@@ -846,8 +864,8 @@ class DifferentialAttention(_Block):
                  rot_base: float, rot_dims: int, scale: float, diff: float, eps: float, max_positions: int, device,
                  dtype, interleaved: bool = True):
         super().__init__(device, dtype)
-        if heads % kv_heads or heads // kv_heads > 16:
-            raise ValueError(f"attention: {heads} query heads over {kv_heads} kv heads (groups of <= 16 supported)")
+        if heads % kv_heads:
+            raise ValueError(f"attention: {heads} query heads do not divide over {kv_heads} kv heads")
         self.layer, self.width, self.H, self.G, self.dim, self.vdim = layer, width, heads, kv_heads, dim, vdim
         self.Hq, self.Hkv, self.group = 2 * heads, 2 * kv_heads, heads // kv_heads
         self.window = int(window) if window and window > 0 else -1

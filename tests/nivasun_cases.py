@@ -64,9 +64,10 @@ def config_b():
 
 def config_c():
     """The whole stack is the loop (start 0, stop = all layers), run twice; five taps; a pair
-    table of one bucket; no convolution at all in the second variant."""
-    return no.make_config([no.latent_layer(mlp=no.moe(4, 2, 8, 8)), no.diff_layer(heads=2, kv_heads=1, mlp=no.moe(3, 2, 6, 0))],
-                          width=16, vocab=29, loop=(0, 2, 2), taps=5, buckets=1, mul_prev=1, mul_cur=1)
+    table of one bucket; a layer with more query heads per kv head than one attention launch takes."""
+    return no.make_config([no.latent_layer(mlp=no.moe(4, 2, 8, 8)), no.diff_layer(heads=2, kv_heads=1, mlp=no.moe(3, 2, 6, 0)),
+                           no.keyed_layer(heads=34, kv_heads=2, dim=4, window=12, rot_dims=2, mlp=None)],
+                          width=16, vocab=29, loop=(0, 3, 2), taps=5, buckets=1, mul_prev=1, mul_cur=1)
 
 
 def config_bf16():

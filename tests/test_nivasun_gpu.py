@@ -127,7 +127,8 @@ def test_router_with_a_logit_bias():
 @pytest.mark.parametrize("kw", [dict(), dict(heads=1, kv_heads=1, dim=8, rot_dims=8),
                                 dict(heads=3, kv_heads=3, dim=10, window=1000, rot_dims=0, scale=1.3),
                                 dict(heads=4, kv_heads=1, dim=70, window=3, rot_dims=6, base=5000.0),
-                                dict(heads=8, kv_heads=2, dim=128, window=40, rot_dims=64, scale=0.09)])
+                                dict(heads=8, kv_heads=2, dim=128, window=40, rot_dims=64, scale=0.09),
+                                dict(heads=34, kv_heads=2, dim=8, window=20, rot_dims=4)])
 def test_key_valued_attention_alone(kw, dt):
     nc.mixer_alone(DEV, dt, no.keyed_layer(**kw), T=70)
 
@@ -136,7 +137,8 @@ def test_key_valued_attention_alone(kw, dt):
 @pytest.mark.parametrize("kw", [dict(), dict(heads=1, kv_heads=1, dim=8, vdim=8, window=1000, rot_dims=8, diff=0.0),
                                 dict(heads=4, kv_heads=1, dim=5, vdim=7, window=6, rot_dims=2, scale=0.9, diff=0.8),
                                 dict(heads=2, kv_heads=2, dim=36, vdim=70, window=1, rot_dims=0),
-                                dict(heads=8, kv_heads=2, dim=64, vdim=128, window=40, rot_dims=32, scale=0.12)])
+                                dict(heads=8, kv_heads=2, dim=64, vdim=128, window=40, rot_dims=32, scale=0.12),
+                                dict(heads=17, kv_heads=1, dim=6, vdim=4, window=20)])
 def test_differential_attention_alone(kw, dt):
     nc.mixer_alone(DEV, dt, no.diff_layer(**kw), T=70)
 
