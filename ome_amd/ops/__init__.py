@@ -1864,6 +1864,8 @@ def latent_attn(q, cache, block_tables, tok_row, kv_lens, scale: float, dv: int,
     parts = MLAWorkspace.parts(T, H, DK)
     if (sinks is not None or window > 0) and DK == 576:   # (these run the 16-head kernel: partition as it does)
         parts = MLAWorkspace.parts(T, H, 0)
+    if window > 0:   # at least four 32-key tiles of the window per partition (fewer only move partials around)
+        parts = max(1, min(parts, window // 128))
     if parts > 1 and ws is None:
         ws = MLAWorkspace(q.device)
     call("ome_latent_attn", q.data_ptr(), q.stride(0), cache.data_ptr(), _i32(block_tables).data_ptr(),
