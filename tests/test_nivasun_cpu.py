@@ -148,3 +148,35 @@ def test_incomplete_checkpoint_is_refused(models, tmp_path):
         path = no.write_model(str(tmp_path / gone), cfg, {k: v for k, v in w.items() if k != gone})
         with pytest.raises(ValueError, match=gone.split(".")[-1]):
             nc.make_engine(path, DEV, "float32")
+
+
+def test_trace_replay_command_line(models, tmp_path):
+    """``bin/trace_run`` as a user runs it: JSON steps on standard input (a prompt portion, a mixed
+    step with a second request, single tokens, a request ended and its slot taken by a third), the
+    wanted logits as little-endian fp32 files, one ``done`` line per step."""
+    import json
+    import subprocess
+
+    import numpy as np
+
+    cfg, w, path, cache = models["c"]
+    a, b, c = nc.prompts(cfg, w, [9, 4, 3], seed=21, min_margin=1e-4)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:6], "want": [0, 5]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[6:8], "want": [1]}, {"id": "b", "tokens": b[:3], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[3:], "want": [0]}, {"id": "a", "tokens": a[8:], "want": [0]}], "end": ["a", "b"]},
+             {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [0, 1, 2]}], "end": ["c"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32", "--out",
+                        str(out), "--max-tokens", "64", "--device", "cpu"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [ln for ln in p.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(4)]
+    V = cfg["vocab"]
+    want = {k: no.forward(cfg, w, t) for k, t in (("a", a), ("b", b), ("c", c))}
+    rows = {0: [("a", 0), ("a", 5)], 1: [("a", 7)], 2: [("b", 3), ("a", 8)], 3: [("c", 0), ("c", 1), ("c", 2)]}
+    for n, rr in rows.items():
+        got = torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, V).copy())
+        assert got.shape[0] == len(rr)
+        for j, (rid, pos) in enumerate(rr):
+            assert nc.logit_errors(got[j:j + 1], want[rid][pos:pos + 1]).max().item() < 2e-4, (n, rid, pos)
