@@ -47,8 +47,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ lo
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
     const int e = lane + 64 * i;
-    v[i] = e < E ? (float)row[e] + (logit_bias ? logit_bias[e] : 0.f) : OME_NEG_INF;   // (a bias of the logits
-    mx = fmaxf(mx, v[i]);                                                               // counts in the scores)
+    // (logit_bias: a router bias that is part of the logits, so it counts in the scores and weights)
+    v[i] = e < E ? (float)row[e] + (logit_bias ? logit_bias[e] : 0.f) : OME_NEG_INF;
+    mx = fmaxf(mx, v[i]);
   }
   mx = wave_max(mx);
   float sum = 0.f;
